@@ -1,0 +1,383 @@
+#include "emit_hip.h"
+
+#include <cmath>
+#include <cstdio>
+#include <sstream>
+#include <stdexcept>
+
+namespace spnc_hip {
+
+namespace {
+
+struct Emitter {
+  const Graph& g;
+  const CompileOptions& o;
+  bool logSpace;
+  bool f64;
+  bool log2Dom;
+  double scale;  // multiplies natural-log constants (log2(e) in the log2 domain)
+  std::ostringstream body;
+  std::vector<double> tablePool;
+  std::vector<uint32_t> tableOffset;   // per node
+  std::vector<uint32_t> featTableLen;  // per feature: longest table of any leaf on it (0 = none)
+  std::vector<bool> featGauss;         // per feature: used by a Gaussian leaf
+  std::vector<bool> featUsed;
+  std::vector<bool> featPrepared;
+  bool vectorRows = true;
+
+  Emitter(const Graph& graph, const CompileOptions& opts) : g(graph), o(opts) {
+    logSpace = o.useLogSpace;
+    f64 = !logSpace || o.computeType == ComputeType::F64;
+    log2Dom = logSpace && !f64 && o.log2Domain;
+    scale = log2Dom ? 1.4426950408889634074 : 1.0;
+  }
+
+  std::string lit(double v) const {
+    if (std::isnan(v)) return f64 ? "__builtin_nan(\"\")" : "__builtin_nanf(\"\")";
+    if (std::isinf(v)) {
+      const char* inf = f64 ? "__builtin_huge_val()" : "__builtin_huge_valf()";
+      return v < 0 ? std::string("(-") + inf + ")" : std::string(inf);
+    }
+    char buf[64];
+    if (f64) {
+      std::snprintf(buf, sizeof(buf), "%a", v);
+    } else {
+      std::snprintf(buf, sizeof(buf), "%af", double(float(v)));
+    }
+    std::string s(buf);
+    return v < 0 ? "(" + s + ")" : s;
+  }
+
+  // log of a probability / weight, moved to the kernel's domain. Logs are taken in double and
+  // rounded once to the compute type, as the reference does for its constants
+  // (mlir/lib/Conversion/HiSPNtoLoSPN/NodePatterns.cpp:56-62,
+  //  mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:120-138).
+  double logConst(double p) const { return p > 0 ? std::log(p) * scale : -INFINITY; }
+
+  static std::string v(uint32_t i) { return "v" + std::to_string(i); }
+
+  template <typename Leaf, typename Comb>
+  std::string tree(size_t lo, size_t hi, Leaf leaf, Comb comb) const {
+    // Balanced binary tree with pivot ceil(k/2), left subtree first
+    // (mlir/lib/Conversion/HiSPNtoLoSPN/NodePatterns.cpp:17-40,49-88).
+    size_t k = hi - lo;
+    if (k == 1) return leaf(lo);
+    if (k == 2) return comb(leaf(lo), leaf(lo + 1));
+    size_t pivot = lo + (k + 1) / 2;
+    return comb(tree(lo, pivot, leaf, comb), tree(pivot, hi, leaf, comb));
+  }
+
+  void prepare() {
+    featTableLen.assign(g.numFeatures, 0);
+    featGauss.assign(g.numFeatures, false);
+    featUsed.assign(g.numFeatures, false);
+    featPrepared.assign(g.numFeatures, false);
+    for (const auto& n : g.nodes) {
+      if (n.kind == NodeKind::Gaussian) {
+        featGauss[n.feature] = true;
+        featUsed[n.feature] = true;
+      } else if (n.kind == NodeKind::Categorical || n.kind == NodeKind::Histogram) {
+        featTableLen[n.feature] = std::max<uint32_t>(featTableLen[n.feature], uint32_t(n.table.size()));
+        featUsed[n.feature] = true;
+      }
+    }
+    // Table pool: every table leaf on feature f owns L_f + 2 entries: its own values, then
+    // "impossible" (log 0 / 0) up to index L_f for out-of-range inputs, then the marginal
+    // value (log 1 / 1) at L_f + 1 for NaN inputs. The index is clamped once per feature.
+    tableOffset.assign(g.nodes.size(), 0);
+    for (size_t i = 0; i < g.nodes.size(); ++i) {
+      const auto& n = g.nodes[i];
+      if (n.kind != NodeKind::Categorical && n.kind != NodeKind::Histogram) continue;
+      uint32_t L = featTableLen[n.feature];
+      tableOffset[i] = uint32_t(tablePool.size());
+      for (uint32_t j = 0; j <= L; ++j) {
+        double p = j < n.table.size() ? n.table[j] : 0.0;
+        tablePool.push_back(logSpace ? logConst(p) : p);
+      }
+      tablePool.push_back(logSpace ? 0.0 : 1.0);
+    }
+  }
+
+  // Emitted right before the first leaf that reads feature f, so that for wide rows the load
+  // sits next to its first use instead of at the top of a very long basic block.
+  void emitFeaturePrep(uint32_t f) {
+    const bool isFloat = g.ftype.isFloat;
+    {
+      if (featPrepared[f]) return;
+      featPrepared[f] = true;
+      std::string x = "x[" + std::to_string(f) + "]";
+      if (!vectorRows) {
+        body << "  const feat_t x" << f << " = __builtin_nontemporal_load(row + " << f << ");\n";
+        x = "x" + std::to_string(f);
+      }
+      if (featGauss[f]) body << "  const real_t g" << f << " = (real_t)" << x << ";\n";
+      if (featTableLen[f]) {
+        uint32_t L = featTableLen[f];
+        if (isFloat) {
+          // fptoui-style truncation, guarded: anything outside [0, L) selects the "impossible" entry.
+          body << "  unsigned t" << f << " = (" << x << " > (feat_t)-1 && " << x << " < (feat_t)" << L << ") ? (unsigned)"
+               << x << " : " << L << "u;\n";
+          if (g.supportMarginal) body << "  t" << f << " = (" << x << " != " << x << ") ? " << (L + 1) << "u : t" << f << ";\n";
+        } else {
+          body << "  const unsigned t" << f << " = (" << x << " < (feat_t)" << L << ") ? (unsigned)" << x << " : " << L
+               << "u;\n";
+        }
+      }
+    }
+  }
+
+  std::string expOf(const std::string& a) const {
+    if (f64) return "exp(" + a + ")";
+    return log2Dom ? "__builtin_amdgcn_exp2f(" + a + ")" : "expf(" + a + ")";
+  }
+  std::string logOf(const std::string& a) const {
+    if (f64) return "log(" + a + ")";
+    return log2Dom ? "__builtin_amdgcn_logf(" + a + ")" : "logf(" + a + ")";
+  }
+  std::string maxOf(const std::string& a, const std::string& b) const {
+    return std::string(f64 ? "__builtin_fmax(" : "__builtin_fmaxf(") + a + ", " + b + ")";
+  }
+
+  void emitLeafMarginal(uint32_t i, const std::string& expr) {
+    const auto& n = g.nodes[i];
+    if (g.supportMarginal) {
+      std::string x = "g" + std::to_string(n.feature);
+      body << "  const real_t " << v(i) << " = (" << x << " != " << x << ") ? " << lit(logSpace ? 0.0 : 1.0) << " : (" << expr
+           << ");\n";
+    } else {
+      body << "  const real_t " << v(i) << " = " << expr << ";\n";
+    }
+  }
+
+  void emitNode(uint32_t i) {
+    const auto& n = g.nodes[i];
+    if (n.kind != NodeKind::Product && n.kind != NodeKind::Sum) emitFeaturePrep(n.feature);
+    switch (n.kind) {
+      case NodeKind::Gaussian: {
+        // log: coef + (x-mean)^2 * den with coef = -ln(sd) - ln(2 pi)/2, den = -1/(2 sd^2)
+        // (mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:306-374); linear: coef' * exp((x-mean)^2 * den)
+        // with coef' = 1/sqrt(2 pi sd^2) (same file :242-304).
+        std::string x = "g" + std::to_string(n.feature);
+        double den = -(1.0 / (2.0 * n.stddev * n.stddev));
+        std::string d = "(" + x + " - " + lit(n.mean) + ")";
+        if (logSpace) {
+          double coef = -std::log(n.stddev) + -0.5 * std::log(2 * M_PI);
+          emitLeafMarginal(i, lit(coef * scale) + " + (" + d + " * " + d + ") * " + lit(den * scale));
+        } else {
+          double coef = 1.0 / std::sqrt(2.0 * M_PI * n.stddev * n.stddev);
+          emitLeafMarginal(i, lit(coef) + " * exp((" + d + " * " + d + ") * " + lit(den) + ")");
+        }
+        break;
+      }
+      case NodeKind::Categorical:
+      case NodeKind::Histogram:
+        body << "  const real_t " << v(i) << " = tab[" << tableOffset[i] << "u + t" << n.feature << "];\n";
+        break;
+      case NodeKind::Product: {
+        const char* op = logSpace ? " + " : " * ";
+        std::string e = tree(
+            0, n.children.size(), [&](size_t k) { return v(n.children[k]); },
+            [&](const std::string& a, const std::string& b) { return "(" + a + op + b + ")"; });
+        body << "  const real_t " << v(i) << " = " << e << ";\n";
+        break;
+      }
+      case NodeKind::Sum:
+        emitSum(i);
+        break;
+    }
+  }
+
+  void emitSum(uint32_t i) {
+    const auto& n = g.nodes[i];
+    size_t k = n.children.size();
+    if (!logSpace) {
+      std::string e = tree(
+          0, k, [&](size_t j) { return "(" + v(n.children[j]) + " * " + lit(n.weights[j]) + ")"; },
+          [&](const std::string& a, const std::string& b) { return "(" + a + " + " + b + ")"; });
+      body << "  const real_t " << v(i) << " = " << e << ";\n";
+      return;
+    }
+    auto term = [&](size_t j) { return "(" + v(n.children[j]) + " + " + lit(logConst(n.weights[j])) + ")"; };
+    if (k == 1) {
+      body << "  const real_t " << v(i) << " = " << term(0) << ";\n";
+      return;
+    }
+    std::string p = "s" + std::to_string(i) + "_";
+    if (o.sumForm == SumForm::Pairwise) {
+      // a + log1p(exp(b - a)) with a the larger operand, over the reference's balanced tree
+      // (mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:216-240).
+      unsigned tmp = 0;
+      std::string e = tree(
+          0, k,
+          [&](size_t j) {
+            std::string name = p + "y" + std::to_string(j);
+            body << "  const real_t " << name << " = " << term(j) << ";\n";
+            return name;
+          },
+          [&](const std::string& a, const std::string& b) {
+            std::string name = p + "t" + std::to_string(tmp++);
+            body << "  const real_t " << name << " = spn_logadd(" << a << ", " << b << ");\n";
+            return name;
+          });
+      body << "  const real_t " << v(i) << " = " << e << ";\n";
+      return;
+    }
+    // n-ary max-shifted log-sum-exp: m = max_j y_j, m + log(sum_j exp(y_j - m)).
+    for (size_t j = 0; j < k; ++j) body << "  const real_t " << p << "y" << j << " = " << term(j) << ";\n";
+    if (k == 2) {
+      // log(1 + exp(-|y0 - y1|)): the larger term contributes exp(0) = 1 exactly.
+      std::string absf = f64 ? "__builtin_fabs" : "__builtin_fabsf";
+      body << "  const real_t " << v(i) << " = " << maxOf(p + "y0", p + "y1") << " + "
+           << logOf(lit(1.0) + " + " + expOf("-" + absf + "(" + p + "y0 - " + p + "y1)")) << ";\n";
+      return;
+    }
+    std::string m = tree(
+        0, k, [&](size_t j) { return p + "y" + std::to_string(j); },
+        [&](const std::string& a, const std::string& b) { return maxOf(a, b); });
+    body << "  const real_t " << p << "m = " << m << ";\n";
+    std::string s = tree(
+        0, k, [&](size_t j) { return expOf(p + "y" + std::to_string(j) + " - " + p + "m"); },
+        [&](const std::string& a, const std::string& b) { return "(" + a + " + " + b + ")"; });
+    body << "  const real_t " << v(i) << " = " << p << "m + " << logOf(s) << ";\n";
+  }
+};
+
+unsigned pickVectorBytes(unsigned rowBytes, unsigned elemBytes) {
+  for (unsigned vb : {16u, 8u, 4u, 2u, 1u})
+    if (vb >= elemBytes && rowBytes % vb == 0) return vb;
+  return elemBytes;
+}
+
+}  // namespace
+
+JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
+  Emitter e(g, o);
+  e.prepare();
+  JitSource js;
+  js.entry = "spn_kernel";
+  js.blockSize = unsigned(o.blockSize);
+  js.bytesPerResult = e.f64 ? 8 : 4;
+  js.tableEntries = unsigned(e.tablePool.size());
+  const unsigned realBytes = e.f64 ? 8 : 4;
+  js.tablesInLds = js.tableEntries > 0 && size_t(js.tableEntries) * realBytes <= 48 * 1024;
+
+  const unsigned F = g.numFeatures;
+  const unsigned eb = g.ftype.bytes;
+  const unsigned rowBytes = F * eb;
+  // Short rows are fetched with the widest vector loads their size allows, all samples of a
+  // lane up front; wide rows are read feature by feature next to the first use.
+  e.vectorRows = rowBytes <= 512;
+  const unsigned vb = e.vectorRows ? pickVectorBytes(rowBytes, eb) : eb;
+  const unsigned vw = vb / eb;
+  js.inputAlign = vb;
+
+  unsigned U = unsigned(o.samplesPerLane);
+  if (U == 0) {
+    size_t work = g.nodes.size() + g.stats.sumTerms;
+    U = work <= 48 ? 4 : (work <= 400 ? 2 : 1);
+  }
+  if (!e.vectorRows) U = 1;
+  js.samplesPerLane = U;
+
+  std::ostringstream s;
+  s << "// generated by spnc-hip for SPN '" << g.name << "': " << g.nodes.size() << " nodes, " << F << " features\n";
+  s << "typedef " << (e.f64 ? "double" : "float") << " real_t;\n";
+  s << "typedef " << g.ftype.hipName << " feat_t;\n";
+  if (vw > 1) s << "typedef feat_t rowvec_t __attribute__((ext_vector_type(" << vw << ")));\n";
+  s << "#define SPN_F " << F << "\n#define SPN_BLOCK " << js.blockSize << "\n#define SPN_U " << U << "\n";
+  if (js.tableEntries) {
+    s << "#define SPN_NTAB " << js.tableEntries << "\n";
+    s << "__device__ const real_t spn_tables[SPN_NTAB] = {";
+    for (size_t i = 0; i < e.tablePool.size(); ++i) s << (i ? ", " : "") << (i % 8 == 0 ? "\n  " : "") << e.lit(e.tablePool[i]);
+    s << "};\n";
+  }
+  if (e.logSpace && o.sumForm == SumForm::Pairwise) {
+    s << "static __device__ __forceinline__ real_t spn_logadd(real_t x, real_t y) {\n"
+         "  const bool gt = x > y;\n  const real_t a = gt ? x : y;\n  const real_t b = gt ? y : x;\n";
+    if (e.f64) s << "  return a + log1p(exp(b - a));\n";
+    else if (e.log2Dom) s << "  return a + __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(b - a));\n";
+    else s << "  return a + log1pf(expf(b - a));\n";
+    s << "}\n";
+  }
+
+  if (e.vectorRows) {
+    s << "static __device__ __forceinline__ void spn_load_row(const feat_t* __restrict__ in, unsigned long long i, feat_t (&x)[SPN_F]) {\n";
+    if (vw == 1) {
+      s << "  const feat_t* p = in + i * SPN_F;\n";
+      for (unsigned f = 0; f < F; ++f)
+        if (e.featUsed[f]) s << "  x[" << f << "] = __builtin_nontemporal_load(p + " << f << ");\n";
+    } else {
+      s << "  const rowvec_t* p = reinterpret_cast<const rowvec_t*>(in + i * SPN_F);\n";
+    }
+    for (unsigned c = 0; vw > 1 && c < F / vw; ++c) {
+      bool used = false;
+      for (unsigned k = 0; k < vw; ++k) used = used || e.featUsed[c * vw + k];
+      if (!used) continue;
+      s << "  const rowvec_t r" << c << " = __builtin_nontemporal_load(p + " << c << ");\n";
+      for (unsigned k = 0; k < vw; ++k)
+        if (e.featUsed[c * vw + k]) s << "  x[" << c * vw + k << "] = r" << c << "[" << k << "];\n";
+    }
+    s << "}\n";
+  }
+
+  for (uint32_t i = 0; i < g.nodes.size(); ++i) e.emitNode(i);
+  if (e.vectorRows)
+    s << "static __device__ __forceinline__ real_t spn_eval(const feat_t (&x)[SPN_F], const real_t* __restrict__ tab) {\n";
+  else
+    s << "static __device__ __forceinline__ real_t spn_eval(const feat_t* __restrict__ row, const real_t* __restrict__ tab) {\n";
+  s << e.body.str();
+  std::string root = Emitter::v(g.root());
+  if (!e.logSpace) s << "  return log(" << root << ");\n";
+  else if (e.log2Dom) s << "  return " << root << " * 0x1.62e43p-1f;\n";  // back to natural log: * ln 2
+  else s << "  return " << root << ";\n";
+  s << "}\n";
+
+  s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK) " << js.entry
+    << "(const feat_t* __restrict__ in, real_t* __restrict__ out, unsigned long long n) {\n";
+  if (js.tableEntries && js.tablesInLds) {
+    s << "  __shared__ real_t tab[SPN_NTAB];\n"
+         "  for (unsigned t = threadIdx.x; t < SPN_NTAB; t += SPN_BLOCK) tab[t] = spn_tables[t];\n"
+         "  __syncthreads();\n";
+  } else if (js.tableEntries) {
+    s << "  const real_t* tab = spn_tables;\n";
+  } else {
+    s << "  const real_t* tab = nullptr;\n";
+  }
+  s << "  const unsigned long long tile = (unsigned long long)SPN_BLOCK * SPN_U;\n"
+       "  for (unsigned long long base = blockIdx.x * tile; base < n; base += gridDim.x * tile) {\n";
+  if (U == 1) {
+    s << "    const unsigned long long i = base + threadIdx.x;\n"
+         "    if (i < n) {\n";
+    if (e.vectorRows)
+      s << "      feat_t x[SPN_F];\n"
+           "      spn_load_row(in, i, x);\n"
+           "      __builtin_nontemporal_store(spn_eval(x, tab), out + i);\n";
+    else
+      s << "      __builtin_nontemporal_store(spn_eval(in + i * SPN_F, tab), out + i);\n";
+    s << "    }\n";
+  } else {
+    s << "    if (base + tile <= n) {\n"
+         "      feat_t x[SPN_U][SPN_F];\n"
+         "#pragma unroll\n"
+         "      for (int u = 0; u < SPN_U; ++u) spn_load_row(in, base + (unsigned long long)u * SPN_BLOCK + threadIdx.x, x[u]);\n"
+         "#pragma unroll\n"
+         "      for (int u = 0; u < SPN_U; ++u)\n"
+         "        __builtin_nontemporal_store(spn_eval(x[u], tab), out + base + (unsigned long long)u * SPN_BLOCK + threadIdx.x);\n"
+         "    } else {\n"
+         "      for (int u = 0; u < SPN_U; ++u) {\n"
+         "        const unsigned long long i = base + (unsigned long long)u * SPN_BLOCK + threadIdx.x;\n"
+         "        if (i < n) {\n"
+         "          feat_t x[SPN_F];\n"
+         "          spn_load_row(in, i, x);\n"
+         "          out[i] = spn_eval(x, tab);\n"
+         "        }\n"
+         "      }\n"
+         "    }\n";
+  }
+  s << "  }\n"
+       "}\n";
+  js.source = s.str();
+  return js;
+}
+
+}  // namespace spnc_hip

@@ -1,0 +1,28 @@
+// Generator for the straight-line per-SPN HIP kernel (gfx950, one sample per lane).
+//
+// Replaces, for the HIP target, the reference's LoSPN->GPU lowering and cubin steps
+// (mlir/lib/Conversion/LoSPNtoGPU/*, compiler/src/pipeline/steps/mlir/conversion/CUDA/*):
+// instead of lowering MLIR it prints one HIP C++ translation unit per SPN, which jit.cpp
+// compiles with hipRTC.
+#pragma once
+#include <string>
+
+#include "options.h"
+#include "spn_graph.h"
+
+namespace spnc_hip {
+
+struct JitSource {
+  std::string source;
+  std::string entry;          // extern "C" kernel symbol
+  unsigned blockSize = 256;
+  unsigned samplesPerLane = 1;
+  unsigned inputAlign = 4;    // required byte alignment of the input base pointer
+  unsigned bytesPerResult = 4;
+  unsigned tableEntries = 0;  // entries of the leaf-table pool (0 = none)
+  bool tablesInLds = false;
+};
+
+JitSource emitHipSource(const Graph& g, const CompileOptions& o);
+
+}  // namespace spnc_hip

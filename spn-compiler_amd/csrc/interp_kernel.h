@@ -1,0 +1,36 @@
+// Launch interface of the table-driven interpreter kernel (see interp_kernel.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace spnc_hip {
+
+constexpr unsigned INTERP_BLOCK = 256;
+
+struct InterpLaunch {
+  const uint32_t* code;      // device: instruction stream
+  const void* in;            // device: [n, numFeatures] row-major, feature type below
+  void* out;                 // device: [n] of the compute type
+  unsigned long long n;
+  const void* tables;        // device: leaf-table pool of the compute type
+  void* spill;               // device: [numSpillSlots][gridDim.x * INTERP_BLOCK] of the compute type
+  const uint32_t* staged;    // device: numStaged * 4 words (column, valueSlot, indexSlot, tableLen)
+  uint32_t numStaged;
+  uint32_t numFeatures;
+  uint32_t featureType;      // spnc_hip::FeatureType as integer
+  uint32_t featureMode;      // FEAT_STAGED / FEAT_DIRECT
+  uint32_t ldsSlots;         // slots [0, ldsSlots) live in LDS, the rest in the spill tier
+  uint32_t marginal;         // NaN features marginalise Gaussian leaves
+};
+
+// Enqueues the interpreter on `stream`. ldsBytes = ldsSlots * INTERP_BLOCK * sizeof(compute type).
+hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain, unsigned grid, size_t ldsBytes, hipStream_t stream);
+
+// Largest dynamic LDS size a block of the interpreter may request on the current device.
+hipError_t interpreterMaxLds(bool f64, bool log2Domain, size_t* bytes);
+
+// Resident blocks per CU for a given dynamic LDS size.
+hipError_t interpreterOccupancy(bool f64, bool log2Domain, size_t ldsBytes, int* blocksPerCU);
+
+}  // namespace spnc_hip

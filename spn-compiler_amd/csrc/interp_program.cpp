@@ -1,0 +1,256 @@
+#include "interp_program.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <queue>
+#include <sstream>
+#include <stdexcept>
+
+namespace spnc_hip {
+
+namespace {
+
+constexpr uint32_t NONE = UINT32_MAX;
+
+struct Builder {
+  const Graph& g;
+  InterpProgram& p;
+  double scale;
+  std::ostringstream txt;
+
+  Builder(const Graph& graph, InterpProgram& prog) : g(graph), p(prog) { scale = p.log2Domain ? 1.4426950408889634074 : 1.0; }
+
+  void word(uint32_t w) { p.code.push_back(w); }
+  void real(double v) {
+    if (p.f64) {
+      uint64_t b;
+      std::memcpy(&b, &v, 8);
+      word(uint32_t(b));
+      word(uint32_t(b >> 32));
+    } else {
+      float f = float(v);
+      uint32_t b;
+      std::memcpy(&b, &f, 4);
+      word(b);
+    }
+  }
+  double logConst(double pr) const { return pr > 0 ? std::log(pr) * scale : -INFINITY; }
+};
+
+}  // namespace
+
+InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
+  if (!o.useLogSpace) throw std::runtime_error("The interpreter kernel supports log-space computation only");
+  InterpProgram p;
+  p.f64 = o.computeType == ComputeType::F64;
+  p.log2Domain = !p.f64 && o.log2Domain;
+  Builder b(g, p);
+  const size_t N = g.nodes.size();
+  auto isLeaf = [&](uint32_t i) { return g.nodes[i].kind != NodeKind::Product && g.nodes[i].kind != NodeKind::Sum; };
+  auto isTable = [&](uint32_t i) { return g.nodes[i].kind == NodeKind::Categorical || g.nodes[i].kind == NodeKind::Histogram; };
+
+  // ---- features: which columns feed Gaussian leaves / table leaves, and the table pool ----
+  std::vector<uint32_t> featTableLen(g.numFeatures, 0);
+  std::vector<bool> featGauss(g.numFeatures, false);
+  for (uint32_t i = 0; i < N; ++i) {
+    const auto& n = g.nodes[i];
+    if (n.kind == NodeKind::Gaussian) featGauss[n.feature] = true;
+    else if (isTable(i)) featTableLen[n.feature] = std::max<uint32_t>(featTableLen[n.feature], uint32_t(n.table.size()));
+  }
+  // Same pool layout as the straight-line kernel: L_f + 2 entries per table leaf (values,
+  // "impossible" up to index L_f, marginal value at L_f + 1).
+  std::vector<uint32_t> tableOffset(N, 0);
+  for (uint32_t i = 0; i < N; ++i) {
+    if (!isTable(i)) continue;
+    const auto& n = g.nodes[i];
+    uint32_t L = featTableLen[n.feature];
+    tableOffset[i] = uint32_t(p.tables.size());
+    for (uint32_t j = 0; j <= L; ++j) p.tables.push_back(b.logConst(j < n.table.size() ? n.table[j] : 0.0));
+    p.tables.push_back(0.0);
+  }
+  uint32_t stagedSlots = 0;
+  for (uint32_t f = 0; f < g.numFeatures; ++f) {
+    stagedSlots += (featGauss[f] ? 1 : 0) + (featTableLen[f] ? 1 : 0);
+  }
+  p.featureMode = stagedSlots <= 48 ? FEAT_STAGED : FEAT_DIRECT;
+  std::vector<uint32_t> valueSlotOf(g.numFeatures, NONE), indexSlotOf(g.numFeatures, NONE);
+  uint32_t nextSlot = 0;
+  if (p.featureMode == FEAT_STAGED) {
+    for (uint32_t f = 0; f < g.numFeatures; ++f) {
+      if (!featGauss[f] && !featTableLen[f]) continue;
+      StagedFeature sf{f, NONE, NONE, featTableLen[f]};
+      if (featGauss[f]) sf.valueSlot = valueSlotOf[f] = nextSlot++;
+      if (featTableLen[f]) sf.indexSlot = indexSlotOf[f] = nextSlot++;
+      p.staged.push_back(sf);
+    }
+  } else {
+    p.directTableLen = featTableLen;
+  }
+  p.reservedSlots = nextSlot;
+
+  // ---- instruction selection ----
+  // A leaf whose only consumer is a product is evaluated inside that product. Every other leaf
+  // becomes a one-term product. Sums with identical ordered child lists form a layer.
+  std::vector<uint32_t> soleParent(N, NONE);
+  for (uint32_t i = 0; i < N; ++i)
+    for (uint32_t c : g.nodes[i].children) soleParent[c] = i;
+  std::vector<bool> inlined(N, false);
+  for (uint32_t i = 0; i < N; ++i)
+    if (isLeaf(i) && g.nodes[i].uses == 1 && soleParent[i] != NONE && g.nodes[soleParent[i]].kind == NodeKind::Product)
+      inlined[i] = true;
+
+  struct Instr {
+    InterpOp op;
+    std::vector<uint32_t> defs;  // graph nodes whose values this instruction writes
+    std::vector<uint32_t> srcs;  // graph nodes read from slots
+    uint32_t node;               // representative node (PROD / SUM) or first sum of a layer
+  };
+  std::vector<Instr> instrs;
+  std::map<std::vector<uint32_t>, std::vector<uint32_t>> layerOf;  // child list -> sums over it
+  for (uint32_t i = 0; i < N; ++i)
+    if (g.nodes[i].kind == NodeKind::Sum && g.nodes[i].children.size() >= 2) layerOf[g.nodes[i].children].push_back(i);
+  std::vector<bool> emitted(N, false);
+  for (uint32_t i = 0; i < N; ++i) {
+    if (emitted[i] || inlined[i]) continue;
+    const auto& n = g.nodes[i];
+    if (n.kind == NodeKind::Sum && n.children.size() >= 2) {
+      const std::vector<uint32_t>& group = layerOf[n.children];
+      // Split the group into layers of 8, 4, 2 sums and single sums.
+      size_t pos = 0;
+      while (pos < group.size()) {
+        size_t left = group.size() - pos;
+        size_t m = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+        Instr in{m == 1 ? OP_SUM : OP_SUMLAYER, {}, n.children, group[pos]};
+        for (size_t j = 0; j < m; ++j) {
+          in.defs.push_back(group[pos + j]);
+          emitted[group[pos + j]] = true;
+        }
+        instrs.push_back(std::move(in));
+        pos += m;
+      }
+      continue;
+    }
+    Instr in{n.kind == NodeKind::Sum ? OP_SUM : OP_PROD, {i}, {}, i};
+    if (n.kind == NodeKind::Sum) {
+      in.srcs = n.children;
+    } else if (n.kind == NodeKind::Product) {
+      for (uint32_t c : n.children)
+        if (!inlined[c]) in.srcs.push_back(c);
+    }
+    emitted[i] = true;
+    instrs.push_back(std::move(in));
+  }
+
+  // ---- slot allocation by liveness on the instruction order ----
+  std::vector<uint32_t> lastUse(N, 0);
+  for (uint32_t k = 0; k < instrs.size(); ++k)
+    for (uint32_t s : instrs[k].srcs) lastUse[s] = k;
+  lastUse[g.root()] = uint32_t(instrs.size());  // read by OP_END
+  std::vector<uint32_t> slotOf(N, NONE);
+  std::priority_queue<uint32_t, std::vector<uint32_t>, std::greater<uint32_t>> freeSlots;
+  uint32_t highWater = nextSlot;
+  auto allocSlot = [&]() {
+    if (!freeSlots.empty()) {
+      uint32_t s = freeSlots.top();
+      freeSlots.pop();
+      return s;
+    }
+    return highWater++;
+  };
+
+  auto emitInlineLeaf = [&](uint32_t c) {
+    const auto& leaf = g.nodes[c];
+    if (leaf.kind == NodeKind::Gaussian) {
+      double coef = -std::log(leaf.stddev) + -0.5 * std::log(2 * M_PI);
+      double den = -(1.0 / (2.0 * leaf.stddev * leaf.stddev));
+      b.word(p.featureMode == FEAT_STAGED ? valueSlotOf[leaf.feature] : leaf.feature);
+      b.real(leaf.mean);
+      b.real(coef * b.scale);
+      b.real(den * b.scale);
+    } else {
+      b.word(p.featureMode == FEAT_STAGED ? indexSlotOf[leaf.feature] : leaf.feature);
+      b.word(tableOffset[c]);
+      b.word(featTableLen[leaf.feature]);
+    }
+  };
+
+  for (uint32_t k = 0; k < instrs.size(); ++k) {
+    const Instr& in = instrs[k];
+    // Sources dying here release their slots before the destinations are chosen: every
+    // opcode reads all of its operands before it writes.
+    {
+      std::vector<uint32_t> uniq = in.srcs;
+      std::sort(uniq.begin(), uniq.end());
+      uniq.erase(std::unique(uniq.begin(), uniq.end()), uniq.end());
+      for (uint32_t s : uniq)
+        if (lastUse[s] == k) freeSlots.push(slotOf[s]);
+    }
+    for (uint32_t d : in.defs) slotOf[d] = allocSlot();
+    const auto& n = g.nodes[in.node];
+    switch (in.op) {
+      case OP_PROD: {
+        std::vector<uint32_t> gs, ts;
+        if (isLeaf(in.node)) {
+          (isTable(in.node) ? ts : gs).push_back(in.node);
+        } else {
+          for (uint32_t c : n.children)
+            if (inlined[c]) (isTable(c) ? ts : gs).push_back(c);
+        }
+        b.word(OP_PROD);
+        b.word(slotOf[in.node]);
+        b.word(uint32_t(in.srcs.size()));
+        b.word(uint32_t(gs.size()));
+        b.word(uint32_t(ts.size()));
+        for (uint32_t s : in.srcs) b.word(slotOf[s]);
+        for (uint32_t c : gs) emitInlineLeaf(c);
+        for (uint32_t c : ts) emitInlineLeaf(c);
+        b.txt << "  s" << slotOf[in.node] << " = prod(" << in.srcs.size() << " slots, " << gs.size() << " gaussians, " << ts.size()
+              << " tables)   ; node " << in.node << "\n";
+        break;
+      }
+      case OP_SUM: {
+        uint32_t cnt = uint32_t(n.children.size());
+        b.word(OP_SUM | (cnt << 8));
+        b.word(slotOf[in.node]);
+        for (uint32_t j = 0; j < cnt; ++j) {
+          b.word(slotOf[n.children[j]]);
+          if (cnt == 1) b.real(b.logConst(n.weights[j]));  // single child: value + log weight
+          else b.real(n.weights[j]);
+        }
+        b.txt << "  s" << slotOf[in.node] << " = sum(" << cnt << " terms)   ; node " << in.node << "\n";
+        break;
+      }
+      case OP_SUMLAYER: {
+        uint32_t cnt = uint32_t(n.children.size());
+        uint32_t m = uint32_t(in.defs.size());
+        b.word(OP_SUMLAYER | (cnt << 8));
+        b.word(m);
+        for (uint32_t d : in.defs) b.word(slotOf[d]);
+        for (uint32_t j = 0; j < cnt; ++j) b.word(slotOf[n.children[j]]);
+        for (uint32_t j = 0; j < cnt; ++j)
+          for (uint32_t d : in.defs) b.real(g.nodes[d].weights[j]);
+        b.txt << "  s" << slotOf[in.defs[0]] << ".. = sumlayer(" << m << " sums x " << cnt << " terms)   ; nodes " << in.defs[0] << "..\n";
+        break;
+      }
+      default:
+        break;
+    }
+    // A value nobody reads later (cannot happen for reachable nodes, kept for safety).
+    for (uint32_t d : in.defs)
+      if (d != g.root() && lastUse[d] <= k) freeSlots.push(slotOf[d]);
+  }
+  b.word(OP_END);
+  b.word(slotOf[g.root()]);
+  p.numSlots = highWater;
+  p.numInstructions = uint32_t(instrs.size());
+  std::ostringstream hdr;
+  hdr << "; interpreter program for SPN '" << g.name << "': " << instrs.size() << " instructions, " << p.code.size() << " words, "
+      << p.numSlots << " value slots (" << p.reservedSlots << " staged features), compute " << (p.f64 ? "f64" : "f32")
+      << (p.log2Domain ? " log2-domain" : "") << ", features " << (p.featureMode == FEAT_STAGED ? "staged" : "direct") << "\n";
+  p.listing = hdr.str() + b.txt.str();
+  return p;
+}
+
+}  // namespace spnc_hip

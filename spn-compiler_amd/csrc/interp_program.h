@@ -1,0 +1,53 @@
+// Node program for the table-driven interpreter kernel: the path for SPN DAGs too large to
+// inline as one straight-line kernel. Plays the role the reference's task partitioner plays
+// for large graphs (mlir/lib/Dialect/LoSPN/Passes/LoSPNTaskPartitioner.cpp), with a different
+// mechanism: one resident kernel walks a wave-uniform instruction stream, operands live in
+// per-lane value slots (LDS first, a coalesced global spill tier behind it).
+#pragma once
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "options.h"
+#include "spn_graph.h"
+
+namespace spnc_hip {
+
+// Opcodes (low 8 bits of an instruction's first word; the upper 24 bits hold a count).
+enum InterpOp : uint32_t {
+  OP_END = 0,       // [op][src]                       result = slot src
+  OP_PROD = 1,      // [op][dst][ns][ng][nt] ns*slot, ng*(feat, mean, coef, den), nt*(feat, tableOffset)
+  OP_SUM = 2,       // [op|k<<8][dst] k*(slot, weight)                 one weighted sum
+  OP_SUMLAYER = 3,  // [op|k<<8][M][dst*M] k*slot, k*M weights        M sums over the same k children (M in 2,4,8)
+};
+
+// How leaves obtain their feature value.
+enum FeatureMode : uint32_t {
+  FEAT_STAGED = 0,  // converted once per tile into reserved slots (feat fields hold slot numbers)
+  FEAT_DIRECT = 1,  // read from the input row at each leaf (feat fields hold column numbers)
+};
+
+struct StagedFeature {
+  uint32_t column;
+  uint32_t valueSlot;  // slot of the value converted to the compute type, or UINT32_MAX
+  uint32_t indexSlot;  // slot of the clamped table index (raw u32 bits), or UINT32_MAX
+  uint32_t tableLen;   // clamp bound L: indices >= L select the "impossible" entry, NaN selects L+1
+};
+
+struct InterpProgram {
+  bool f64 = false;
+  bool log2Domain = true;
+  FeatureMode featureMode = FEAT_STAGED;
+  std::vector<uint32_t> code;
+  std::vector<double> tables;          // pool of leaf tables in the kernel's log domain
+  std::vector<uint32_t> directTableLen;  // FEAT_DIRECT: per column clamp bound (0 = none)
+  std::vector<StagedFeature> staged;
+  uint32_t numSlots = 0;      // value slots the program addresses, staged features included
+  uint32_t reservedSlots = 0; // leading slots pinned to staged features
+  uint32_t numInstructions = 0;
+  std::string listing;        // human-readable form, for "dump-ir"
+};
+
+InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o);
+
+}  // namespace spnc_hip

@@ -1,0 +1,491 @@
+#include "kernel.h"
+
+#include <hip/hiprtc.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <stdexcept>
+
+#include "interp_kernel.h"
+
+namespace spnc_hip {
+
+namespace {
+
+[[noreturn]] void fatal(const std::string& m) { throw std::runtime_error(m); }
+
+void hipCheck(hipError_t e, const char* what) {
+  if (e != hipSuccess) fatal(std::string("HIP error in ") + what + ": " + hipGetErrorString(e));
+}
+
+std::vector<char> compileWithHipRtc(const JitSource& js, int optLevel) {
+  hiprtcProgram prog;
+  if (hiprtcCreateProgram(&prog, js.source.c_str(), "spn_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+    fatal("hiprtcCreateProgram failed");
+  std::string opt = "-O" + std::to_string(std::max(0, std::min(3, optLevel)));
+  // Packed-FP32 instruction selection is switched off for all device code of this library.
+  const char* opts[] = {"--offload-arch=gfx950", opt.c_str(),       "-std=c++17",       "-ffp-contract=fast",
+                        "-Xclang",               "-target-feature", "-Xclang",          "-packed-fp32-ops"};
+  hiprtcResult r = hiprtcCompileProgram(prog, int(sizeof(opts) / sizeof(opts[0])), opts);
+  if (r != HIPRTC_SUCCESS) {
+    size_t ls = 0;
+    hiprtcGetProgramLogSize(prog, &ls);
+    std::string log(ls, '\0');
+    if (ls) hiprtcGetProgramLog(prog, &log[0]);
+    hiprtcDestroyProgram(&prog);
+    fatal("COMPILATION ERROR: hipRTC failed: " + log);
+  }
+  size_t cs = 0;
+  hiprtcGetCodeSize(prog, &cs);
+  std::vector<char> code(cs);
+  hiprtcGetCode(prog, code.data());
+  hiprtcDestroyProgram(&prog);
+  return code;
+}
+
+// ---- kernel file: magic, then tagged little-endian fields ----
+const char kMagic[8] = {'S', 'P', 'N', 'C', 'H', 'I', 'P', 1};
+
+struct Writer {
+  std::vector<char> buf;
+  void u32(uint32_t v) { raw(&v, 4); }
+  void u64(uint64_t v) { raw(&v, 8); }
+  void raw(const void* p, size_t n) { buf.insert(buf.end(), static_cast<const char*>(p), static_cast<const char*>(p) + n); }
+  void str(const std::string& s) {
+    u64(s.size());
+    raw(s.data(), s.size());
+  }
+  template <typename T>
+  void vec(const std::vector<T>& v) {
+    u64(v.size());
+    raw(v.data(), v.size() * sizeof(T));
+  }
+};
+
+struct Reader {
+  const std::vector<char>& buf;
+  size_t pos = 0;
+  explicit Reader(const std::vector<char>& b) : buf(b) {}
+  void raw(void* p, size_t n) {
+    if (n > buf.size() - pos) fatal("RUNTIME ERROR: truncated kernel file");
+    std::memcpy(p, buf.data() + pos, n);
+    pos += n;
+  }
+  uint32_t u32() {
+    uint32_t v;
+    raw(&v, 4);
+    return v;
+  }
+  uint64_t u64() {
+    uint64_t v;
+    raw(&v, 8);
+    return v;
+  }
+  std::string str() {
+    uint64_t n = u64();
+    if (n > buf.size() - pos) fatal("RUNTIME ERROR: truncated kernel file");
+    std::string s(buf.data() + pos, size_t(n));
+    pos += size_t(n);
+    return s;
+  }
+  template <typename T>
+  std::vector<T> vec() {
+    uint64_t n = u64();
+    if (n > (buf.size() - pos) / sizeof(T)) fatal("RUNTIME ERROR: truncated kernel file");
+    std::vector<T> v(static_cast<size_t>(n));
+    raw(v.data(), size_t(n) * sizeof(T));
+    return v;
+  }
+};
+
+std::string makeKernelFilePath() {
+  const char* dir = std::getenv("TMPDIR");
+  std::string tmpl = std::string(dir && *dir ? dir : "/tmp") + "/spnc_hip_XXXXXX.hipk";
+  std::vector<char> path(tmpl.begin(), tmpl.end());
+  path.push_back('\0');
+  int fd = mkstemps(path.data(), 5);
+  if (fd < 0) fatal("COMPILATION ERROR: cannot create kernel file " + tmpl);
+  close(fd);
+  return std::string(path.data());
+}
+
+}  // namespace
+
+std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std::map<std::string, std::string>& options) {
+  CompileOptions o = parseOptions(options);
+  RawQuery q = readQueryFile(queryPath);
+  Graph g = buildGraph(q);
+  std::unique_ptr<Kernel> k(new Kernel());
+  k->kernelName_ = g.name;
+  k->batchSize_ = unsigned(std::max(1, g.batchSize));
+  k->numFeatures_ = g.numFeatures;
+  k->bytesPerFeature_ = g.ftype.bytes;
+  k->featureType_ = unsigned(g.ftype.type);
+  k->marginal_ = g.supportMarginal;
+  k->stats_ = g.stats;
+  k->numNodes_ = unsigned(g.nodes.size());
+
+  const uint64_t ops = g.nodes.size() + g.stats.sumTerms + g.stats.productAdds;
+  bool useInterp = o.kernelMode == KernelMode::Interpreter || (o.kernelMode == KernelMode::Auto && ops > uint64_t(std::max(0, o.jitMaxOps)));
+  if (useInterp && !o.useLogSpace) {
+    if (o.kernelMode == KernelMode::Interpreter) fatal("COMPILATION ERROR: the interpreter kernel supports log-space computation only");
+    useInterp = false;
+  }
+  if (useInterp) {
+    k->kind_ = SPNC_HIP_KERNEL_INTERPRETER;
+    k->prog_ = buildInterpProgram(g, o);
+    k->bytesPerResult_ = k->prog_.f64 ? 8 : 4;
+    k->inputAlign_ = g.ftype.bytes;
+    k->text_ = k->prog_.listing;
+  } else {
+    k->kind_ = SPNC_HIP_KERNEL_JIT;
+    JitSource js = emitHipSource(g, o);
+    k->codeObject_ = compileWithHipRtc(js, o.optLevel);
+    k->entry_ = js.entry;
+    k->blockSize_ = js.blockSize;
+    k->samplesPerLane_ = js.samplesPerLane;
+    k->inputAlign_ = js.inputAlign;
+    k->bytesPerResult_ = js.bytesPerResult;
+    k->text_ = std::move(js.source);
+  }
+  if (o.dumpIR) std::cerr << "// *** device code for " << k->kernelName_ << " ***\n" << k->text_ << std::endl;
+  if (o.collectGraphStats) {
+    std::ofstream st(o.graphStatsFile);
+    const GraphStats& s = g.stats;
+    st << "{\"featureCount\": " << g.numFeatures << ", \"sumCount\": " << s.sums << ", \"productCount\": " << s.products
+       << ", \"histogramCount\": " << s.histograms << ", \"categoricalCount\": " << s.categoricals << ", \"gaussianCount\": " << s.gaussians
+       << ", \"innerCount\": " << (s.sums + s.products) << ", \"leafCount\": " << (s.histograms + s.categoricals + s.gaussians)
+       << ", \"maxFanIn\": " << s.maxFanIn << ", \"sumTerms\": " << s.sumTerms << ", \"flopsMin\": " << s.flopsMin
+       << ", \"transMin\": " << s.transMin << "}\n";
+  }
+  k->fileName_ = makeKernelFilePath();
+  k->save(k->fileName_);
+  return k;
+}
+
+void Kernel::save(const std::string& path) const {
+  Writer w;
+  w.raw(kMagic, 8);
+  w.str(kernelName_);
+  w.u32(batchSize_);
+  w.u32(numFeatures_);
+  w.u32(bytesPerFeature_);
+  w.u32(bytesPerResult_);
+  w.u32(featureType_);
+  w.u32(marginal_);
+  w.u32(kind_);
+  w.u32(numNodes_);
+  w.raw(&stats_, sizeof(stats_));
+  w.str(text_);
+  if (kind_ == SPNC_HIP_KERNEL_JIT) {
+    w.vec(codeObject_);
+    w.str(entry_);
+    w.u32(blockSize_);
+    w.u32(samplesPerLane_);
+    w.u32(inputAlign_);
+  } else {
+    w.u32(prog_.f64);
+    w.u32(prog_.log2Domain);
+    w.u32(prog_.featureMode);
+    w.vec(prog_.code);
+    w.vec(prog_.tables);
+    w.vec(prog_.directTableLen);
+    w.u64(prog_.staged.size());
+    for (const auto& s : prog_.staged) {
+      w.u32(s.column);
+      w.u32(s.valueSlot);
+      w.u32(s.indexSlot);
+      w.u32(s.tableLen);
+    }
+    w.u32(prog_.numSlots);
+    w.u32(prog_.reservedSlots);
+    w.u32(prog_.numInstructions);
+  }
+  FILE* f = std::fopen(path.c_str(), "wb");
+  if (!f) fatal("COMPILATION ERROR: cannot write kernel file " + path);
+  size_t n = std::fwrite(w.buf.data(), 1, w.buf.size(), f);
+  std::fclose(f);
+  if (n != w.buf.size()) fatal("COMPILATION ERROR: short write to kernel file " + path);
+}
+
+std::unique_ptr<Kernel> Kernel::load(const std::string& kernelFile) {
+  std::ifstream f(kernelFile, std::ios::binary);
+  if (!f) fatal("RUNTIME ERROR: cannot open kernel file " + kernelFile);
+  std::vector<char> buf((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+  if (buf.size() < 8 || std::memcmp(buf.data(), kMagic, 8) != 0) fatal("RUNTIME ERROR: " + kernelFile + " is not a spnc-hip kernel file");
+  Reader r(buf);
+  r.pos = 8;
+  std::unique_ptr<Kernel> k(new Kernel());
+  k->fileName_ = kernelFile;
+  k->kernelName_ = r.str();
+  k->batchSize_ = r.u32();
+  k->numFeatures_ = r.u32();
+  k->bytesPerFeature_ = r.u32();
+  k->bytesPerResult_ = r.u32();
+  k->featureType_ = r.u32();
+  k->marginal_ = r.u32() != 0;
+  k->kind_ = r.u32();
+  k->numNodes_ = r.u32();
+  r.raw(&k->stats_, sizeof(k->stats_));
+  k->text_ = r.str();
+  if (k->kind_ == SPNC_HIP_KERNEL_JIT) {
+    k->codeObject_ = r.vec<char>();
+    k->entry_ = r.str();
+    k->blockSize_ = r.u32();
+    k->samplesPerLane_ = r.u32();
+    k->inputAlign_ = r.u32();
+  } else if (k->kind_ == SPNC_HIP_KERNEL_INTERPRETER) {
+    k->prog_.f64 = r.u32() != 0;
+    k->prog_.log2Domain = r.u32() != 0;
+    k->prog_.featureMode = FeatureMode(r.u32());
+    k->prog_.code = r.vec<uint32_t>();
+    k->prog_.tables = r.vec<double>();
+    k->prog_.directTableLen = r.vec<uint32_t>();
+    uint64_t ns = r.u64();
+    for (uint64_t i = 0; i < ns; ++i) {
+      StagedFeature s;
+      s.column = r.u32();
+      s.valueSlot = r.u32();
+      s.indexSlot = r.u32();
+      s.tableLen = r.u32();
+      k->prog_.staged.push_back(s);
+    }
+    k->prog_.numSlots = r.u32();
+    k->prog_.reservedSlots = r.u32();
+    k->prog_.numInstructions = r.u32();
+    k->inputAlign_ = k->bytesPerFeature_;
+  } else {
+    fatal("RUNTIME ERROR: unknown kernel kind in " + kernelFile);
+  }
+  return k;
+}
+
+Kernel::~Kernel() { releaseDevice(); }
+
+void Kernel::fillInfo(spnc_hip_info* info) const {
+  std::memset(info, 0, sizeof(*info));
+  std::snprintf(info->file_name, sizeof(info->file_name), "%s", fileName_.c_str());
+  std::snprintf(info->kernel_name, sizeof(info->kernel_name), "%s", kernelName_.c_str());
+  info->query_type = SPNC_HIP_QUERY_JOINT;
+  info->target = SPNC_HIP_TARGET_HIP;
+  info->batch_size = batchSize_;
+  info->num_features = numFeatures_;
+  info->bytes_per_feature = bytesPerFeature_;
+  info->num_results = 1;
+  info->bytes_per_result = bytesPerResult_;
+  std::snprintf(info->dtype, sizeof(info->dtype), "%s", bytesPerResult_ == 8 ? "float64" : "float32");
+  info->kernel_kind = kind_;
+  info->input_alignment = inputAlign_;
+  info->num_nodes = numNodes_;
+  info->num_gaussian = stats_.gaussians;
+  info->num_categorical = stats_.categoricals;
+  info->num_histogram = stats_.histograms;
+  info->num_product = stats_.products;
+  info->num_sum = stats_.sums;
+  info->max_fan_in = stats_.maxFanIn;
+  info->sum_terms = stats_.sumTerms;
+  info->product_adds = stats_.productAdds;
+  info->flops_min = stats_.flopsMin;
+  info->trans_min = stats_.transMin;
+  info->flops_pairwise = stats_.flopsPairwise;
+  info->trans_pairwise = stats_.transPairwise;
+}
+
+void Kernel::ensureDevice() {
+  if (deviceReady_) return;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count == 0) fatal("RUNTIME ERROR: no HIP device available");
+  hipCheck(hipGetDevice(&device_), "hipGetDevice");
+  hipDeviceProp_t prop;
+  hipCheck(hipGetDeviceProperties(&prop, device_), "hipGetDeviceProperties");
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    fatal(std::string("RUNTIME ERROR: kernels are built for gfx950, device is ") + prop.gcnArchName);
+  numCUs_ = prop.multiProcessorCount;
+  if (kind_ == SPNC_HIP_KERNEL_JIT) {
+    hipCheck(hipModuleLoadData(&module_, codeObject_.data()), "hipModuleLoadData");
+    hipCheck(hipModuleGetFunction(&function_, module_, entry_.c_str()), "hipModuleGetFunction");
+    int nb = 0;
+    hipCheck(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&nb, function_, int(blockSize_), 0), "occupancy query");
+    blocksPerCU_ = std::max(1, nb);
+  } else {
+    const size_t rb = prog_.f64 ? 8 : 4;
+    // Value slots in LDS: as many as the program needs, capped so that two blocks fit a CU.
+    int ldsPerCU = 0;
+    hipCheck(hipDeviceGetAttribute(&ldsPerCU, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, device_), "LDS size query");
+    size_t maxBlock = 0;
+    hipCheck(interpreterMaxLds(prog_.f64, prog_.log2Domain, &maxBlock), "LDS limit query");
+    size_t budget = std::min<size_t>(maxBlock, size_t(ldsPerCU) / 2);
+    uint32_t cap = uint32_t(budget / (INTERP_BLOCK * rb));
+    ldsSlots_ = std::min(prog_.numSlots, cap);
+    ldsBytes_ = size_t(ldsSlots_) * INTERP_BLOCK * rb;
+    int nb = 0;
+    hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, ldsBytes_, &nb), "occupancy query");
+    blocksPerCU_ = std::max(1, nb);
+    hipCheck(hipMalloc(&dCode_, prog_.code.size() * 4), "hipMalloc(program)");
+    hipCheck(hipMemcpy(dCode_, prog_.code.data(), prog_.code.size() * 4, hipMemcpyHostToDevice), "program upload");
+    if (!prog_.tables.empty()) {
+      hipCheck(hipMalloc(&dTables_, prog_.tables.size() * rb), "hipMalloc(tables)");
+      if (prog_.f64) {
+        hipCheck(hipMemcpy(dTables_, prog_.tables.data(), prog_.tables.size() * 8, hipMemcpyHostToDevice), "table upload");
+      } else {
+        std::vector<float> t(prog_.tables.begin(), prog_.tables.end());
+        hipCheck(hipMemcpy(dTables_, t.data(), t.size() * 4, hipMemcpyHostToDevice), "table upload");
+      }
+    }
+    if (!prog_.staged.empty()) {
+      std::vector<uint32_t> st;
+      for (const auto& s : prog_.staged) {
+        st.push_back(s.column);
+        st.push_back(s.valueSlot);
+        st.push_back(s.indexSlot);
+        st.push_back(s.tableLen);
+      }
+      hipCheck(hipMalloc(&dStaged_, st.size() * 4), "hipMalloc(staged)");
+      hipCheck(hipMemcpy(dStaged_, st.data(), st.size() * 4, hipMemcpyHostToDevice), "staged upload");
+    }
+    const size_t lanes = size_t(numCUs_) * blocksPerCU_ * INTERP_BLOCK;
+    spillBytes_ = size_t(prog_.numSlots - ldsSlots_) * lanes * rb;
+    if (spillBytes_) hipCheck(hipMalloc(&dSpill_, spillBytes_), "hipMalloc(spill)");
+  }
+  deviceReady_ = true;
+}
+
+void Kernel::releaseDevice() {
+  for (auto& s : stage_) {
+    if (s.stream) (void)hipStreamSynchronize(s.stream);
+    if (s.hIn) (void)hipHostFree(s.hIn);
+    if (s.hOut) (void)hipHostFree(s.hOut);
+    if (s.dIn) (void)hipFree(s.dIn);
+    if (s.dOut) (void)hipFree(s.dOut);
+    if (s.stream) (void)hipStreamDestroy(s.stream);
+    s = Stage();
+  }
+  stageRows_ = 0;
+  if (kernelDone_) (void)hipEventDestroy(kernelDone_);
+  kernelDone_ = nullptr;
+  if (dCode_) (void)hipFree(dCode_);
+  if (dTables_) (void)hipFree(dTables_);
+  if (dStaged_) (void)hipFree(dStaged_);
+  if (dSpill_) (void)hipFree(dSpill_);
+  dCode_ = nullptr;
+  dTables_ = nullptr;
+  dStaged_ = nullptr;
+  dSpill_ = nullptr;
+  if (module_) (void)hipModuleUnload(module_);
+  module_ = nullptr;
+  function_ = nullptr;
+  deviceReady_ = false;
+}
+
+void Kernel::launch(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
+  if (n == 0) return;
+  if (reinterpret_cast<uintptr_t>(dIn) % inputAlign_ != 0)
+    fatal("RUNTIME ERROR: input pointer must be aligned to " + std::to_string(inputAlign_) + " bytes");
+  if (reinterpret_cast<uintptr_t>(dOut) % bytesPerResult_ != 0) fatal("RUNTIME ERROR: output pointer is misaligned");
+  if (kind_ == SPNC_HIP_KERNEL_JIT) {
+    const size_t tile = size_t(blockSize_) * samplesPerLane_;
+    const size_t tiles = (n + tile - 1) / tile;
+    const unsigned grid = unsigned(std::min<size_t>(tiles, size_t(numCUs_) * blocksPerCU_));
+    unsigned long long n64 = n;
+    void* args[] = {(void*)&dIn, (void*)&dOut, (void*)&n64};
+    hipCheck(hipModuleLaunchKernel(function_, grid, 1, 1, blockSize_, 1, 1, 0, stream, args, nullptr), "kernel launch");
+  } else {
+    const size_t tiles = (n + INTERP_BLOCK - 1) / INTERP_BLOCK;
+    const unsigned grid = unsigned(std::min<size_t>(tiles, size_t(numCUs_) * blocksPerCU_));
+    InterpLaunch a;
+    a.code = dCode_;
+    a.in = dIn;
+    a.out = dOut;
+    a.n = n;
+    a.tables = dTables_;
+    a.spill = dSpill_;
+    a.staged = dStaged_;
+    a.numStaged = uint32_t(prog_.staged.size());
+    a.numFeatures = numFeatures_;
+    a.featureType = featureType_;
+    a.featureMode = prog_.featureMode;
+    a.ldsSlots = ldsSlots_;
+    a.marginal = marginal_ ? 1u : 0u;
+    hipCheck(launchInterpreter(a, prog_.f64, prog_.log2Domain, grid, ldsBytes_, stream), "interpreter launch");
+  }
+}
+
+void Kernel::executeDevice(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(mu_);
+  ensureDevice();
+  launch(n, dIn, dOut, stream);
+}
+
+void Kernel::ensureStaging(size_t rows) {
+  if (rows <= stageRows_) return;
+  for (auto& s : stage_) {
+    if (s.hIn) (void)hipHostFree(s.hIn);
+    if (s.hOut) (void)hipHostFree(s.hOut);
+    if (s.dIn) (void)hipFree(s.dIn);
+    if (s.dOut) (void)hipFree(s.dOut);
+    s.hIn = s.hOut = s.dIn = s.dOut = nullptr;
+    const size_t inBytes = rows * numFeatures_ * bytesPerFeature_, outBytes = rows * bytesPerResult_;
+    hipCheck(hipHostMalloc(&s.hIn, inBytes, hipHostMallocDefault), "hipHostMalloc(input staging)");
+    hipCheck(hipHostMalloc(&s.hOut, outBytes, hipHostMallocDefault), "hipHostMalloc(output staging)");
+    hipCheck(hipMalloc(&s.dIn, inBytes), "hipMalloc(input)");
+    hipCheck(hipMalloc(&s.dOut, outBytes), "hipMalloc(output)");
+    if (!s.stream) hipCheck(hipStreamCreate(&s.stream), "hipStreamCreate");
+  }
+  if (!kernelDone_) hipCheck(hipEventCreateWithFlags(&kernelDone_, hipEventDisableTiming), "hipEventCreate");
+  stageRows_ = rows;
+}
+
+void Kernel::execute(size_t n, const void* in, void* out) {
+  std::lock_guard<std::mutex> lock(mu_);
+  ensureDevice();
+  if (n == 0) return;
+  if (!in || !out) fatal("RUNTIME ERROR: null input or output buffer");
+  const size_t rowBytes = size_t(numFeatures_) * bytesPerFeature_;
+  // Chunks of about 32 MiB of input, two in flight: copy-in, kernel and copy-out of one
+  // chunk overlap the host-side staging of the next.
+  size_t chunk = std::max<size_t>(4096, (size_t(32) << 20) / std::max<size_t>(1, rowBytes));
+  chunk = std::min(chunk, n);
+  ensureStaging(chunk);
+  auto drain = [&](Stage& s) {
+    if (!s.pendingRows) return;
+    hipCheck(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
+    std::memcpy(static_cast<char*>(out) + s.pendingOffset * bytesPerResult_, s.hOut, s.pendingRows * bytesPerResult_);
+    s.pendingRows = 0;
+  };
+  size_t done = 0;
+  unsigned turn = 0;
+  try {
+    while (done < n) {
+      Stage& s = stage_[turn & 1];
+      drain(s);
+      const size_t rows = std::min(chunk, n - done);
+      std::memcpy(s.hIn, static_cast<const char*>(in) + done * rowBytes, rows * rowBytes);
+      hipCheck(hipMemcpyAsync(s.dIn, s.hIn, rows * rowBytes, hipMemcpyHostToDevice, s.stream), "input copy");
+      // Kernels of successive chunks run one after the other (they share the spill buffer);
+      // only the copies overlap them.
+      if (turn) hipCheck(hipStreamWaitEvent(s.stream, kernelDone_, 0), "hipStreamWaitEvent");
+      launch(rows, s.dIn, s.dOut, s.stream);
+      hipCheck(hipEventRecord(kernelDone_, s.stream), "hipEventRecord");
+      hipCheck(hipMemcpyAsync(s.hOut, s.dOut, rows * bytesPerResult_, hipMemcpyDeviceToHost, s.stream), "output copy");
+      s.pendingRows = rows;
+      s.pendingOffset = done;
+      done += rows;
+      ++turn;
+    }
+    drain(stage_[0]);
+    drain(stage_[1]);
+  } catch (...) {
+    for (auto& s : stage_) {
+      if (s.stream) (void)hipStreamSynchronize(s.stream);
+      s.pendingRows = 0;
+    }
+    throw;
+  }
+}
+
+}  // namespace spnc_hip

@@ -1,0 +1,102 @@
+#include "options.h"
+
+#include <algorithm>
+#include <cctype>
+#include <set>
+#include <stdexcept>
+
+namespace spnc_hip {
+
+namespace {
+
+bool parseBool(const std::string& v) {
+  std::string s = v;
+  std::transform(s.begin(), s.end(), s.begin(), [](unsigned char c) { return char(std::tolower(c)); });
+  return s == "true" || s == "yes";
+}
+
+int parseInt(const std::string& key, const std::string& v) {
+  try {
+    size_t pos = 0;
+    int r = std::stoi(v, &pos);
+    if (pos != v.size()) throw std::invalid_argument(v);
+    return r;
+  } catch (const std::exception&) {
+    throw std::runtime_error("Could not parse option value " + v + " for " + key);
+  }
+}
+
+// Options of the reference that steer only its CPU / MLIR / CUDA pipelines.
+const std::set<std::string>& ignoredKeys() {
+  static const std::set<std::string> k = {
+      "irOptLevel", "mcOptLevel", "cpu-vectorize", "vector-library", "use-shuffle", "slp-max-attempts",
+      "slp-max-successful-iterations", "slp-max-node-size", "slp-max-look-ahead", "slp-reorder-dfs",
+      "slp-allow-duplicate-elements", "slp-allow-topological-mixing", "slp-use-xor-chains", "search-paths",
+      "opt-repr", "stopAfter"};
+  return k;
+}
+
+}  // namespace
+
+CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
+  CompileOptions o;
+  bool haveTarget = false;
+  for (const auto& e : kv) {
+    const std::string& key = e.first;
+    const std::string& val = e.second;
+    if (key == "target") {
+      if (val != "HIP") throw std::runtime_error("Target was '" + val + "', but this compiler only supports target 'HIP'");
+      haveTarget = true;
+    } else if (key == "use-log-space") {
+      o.useLogSpace = parseBool(val);
+    } else if (key == "gpu-shared-mem") {
+      o.gpuSharedMem = parseBool(val);
+    } else if (key == "dump-ir") {
+      o.dumpIR = parseBool(val);
+    } else if (key == "collect-graph-stats") {
+      o.collectGraphStats = parseBool(val);
+    } else if (key == "graph-stats-file") {
+      o.graphStatsFile = val;
+    } else if (key == "maxTaskSize") {
+      o.maxTaskSize = parseInt(key, val);
+    } else if (key == "optLevel") {
+      o.optLevel = parseInt(key, val);
+    } else if (key == "delete-temps") {
+      o.deleteTemps = parseBool(val);
+    } else if (key == "hip-compute-type") {
+      if (val == "float32") o.computeType = ComputeType::F32;
+      else if (val == "float64") o.computeType = ComputeType::F64;
+      else throw std::runtime_error("Could not parse option value " + val + " for " + key);
+    } else if (key == "hip-kernel") {
+      if (val == "auto") o.kernelMode = KernelMode::Auto;
+      else if (val == "jit") o.kernelMode = KernelMode::Jit;
+      else if (val == "interpreter") o.kernelMode = KernelMode::Interpreter;
+      else throw std::runtime_error("Could not parse option value " + val + " for " + key);
+    } else if (key == "hip-sum-form") {
+      if (val == "nary") o.sumForm = SumForm::Nary;
+      else if (val == "pairwise") o.sumForm = SumForm::Pairwise;
+      else throw std::runtime_error("Could not parse option value " + val + " for " + key);
+    } else if (key == "hip-log2-domain") {
+      o.log2Domain = parseBool(val);
+    } else if (key == "hip-samples-per-lane") {
+      o.samplesPerLane = parseInt(key, val);
+      if (o.samplesPerLane < 0 || o.samplesPerLane > 16) throw std::runtime_error("hip-samples-per-lane must be in [0,16]");
+    } else if (key == "hip-jit-max-ops") {
+      o.jitMaxOps = parseInt(key, val);
+    } else if (key == "hip-block-size") {
+      o.blockSize = parseInt(key, val);
+      if (o.blockSize != 64 && o.blockSize != 128 && o.blockSize != 256 && o.blockSize != 512)
+        throw std::runtime_error("hip-block-size must be 64, 128, 256 or 512");
+    } else if (ignoredKeys().count(key)) {
+      // accepted for compatibility, no effect on the HIP target
+    } else {
+      throw std::runtime_error("Unknown compile option " + key);
+    }
+  }
+  if (!haveTarget) throw std::runtime_error("Could not verify configuration constraints!");
+  if (o.collectGraphStats == false && kv.count("graph-stats-file"))
+    throw std::runtime_error("Could not verify configuration constraints!");
+  return o;
+}
+
+}  // namespace spnc_hip

@@ -1,0 +1,38 @@
+// String-keyed compile options for the HIP target.
+//
+// Keeps the reference's option names and parsing rules (compiler/src/option/GlobalOptions.cpp:14-75;
+// booleans are true for "true"/"yes" in any case, compiler/src/option/Options.cpp:78-82; an unknown key
+// is fatal, compiler/src/option/Options.h:222-224; "target" is required). Options that only steer the
+// reference's CPU/MLIR pipeline are accepted and ignored; options prefixed "hip-" are new.
+#pragma once
+#include <map>
+#include <string>
+
+namespace spnc_hip {
+
+enum class KernelMode { Auto, Jit, Interpreter };
+enum class SumForm { Nary, Pairwise };
+enum class ComputeType { F32, F64 };
+
+struct CompileOptions {
+  bool useLogSpace = false;     // "use-log-space" (reference default false; the Python front passes true)
+  bool gpuSharedMem = true;     // "gpu-shared-mem": stage the input tile through LDS
+  bool dumpIR = false;          // "dump-ir": print the generated device source / program
+  bool collectGraphStats = false;
+  std::string graphStatsFile = "/tmp/stats.json";
+  int maxTaskSize = -1;
+  int optLevel = 3;
+  bool deleteTemps = true;
+  ComputeType computeType = ComputeType::F32;  // "hip-compute-type": float32 | float64 (log-space only)
+  KernelMode kernelMode = KernelMode::Auto;    // "hip-kernel": auto | jit | interpreter
+  SumForm sumForm = SumForm::Nary;             // "hip-sum-form": nary | pairwise
+  bool log2Domain = true;                      // "hip-log2-domain": carry log2 values in f32 kernels
+  int samplesPerLane = 0;                      // "hip-samples-per-lane": 0 = choose from SPN size
+  int jitMaxOps = 20000;                       // "hip-jit-max-ops": above this, auto picks the interpreter
+  int blockSize = 256;                         // "hip-block-size"
+};
+
+// Throws std::runtime_error("Unknown compile option <key>") etc.
+CompileOptions parseOptions(const std::map<std::string, std::string>& kv);
+
+}  // namespace spnc_hip

@@ -1,0 +1,353 @@
+#include "spn_graph.h"
+
+#include <algorithm>
+#include <cmath>
+#include <map>
+#include <stdexcept>
+#include <unordered_map>
+
+#include "capnp_reader.h"
+
+namespace spnc_hip {
+
+namespace {
+
+[[noreturn]] void fatal(const std::string& msg) { throw std::runtime_error(msg); }
+
+// Field offsets follow the standard Cap'n Proto layout of the reference's schema
+// (xspn/xspn/serialization/binary/capnproto/spflow.capnp:27-102).
+RawNode decodeNode(const capnp::StructReader& s) {
+  RawNode n;
+  n.id = s.get<int32_t>(0);
+  n.root = s.getBool(32);
+  uint16_t which = s.get<uint16_t>(6);
+  capnp::StructReader body = s.getStruct(0);
+  switch (which) {
+    case 0:
+      n.kind = NodeKind::Product;
+      n.children = body.getList(0).toVector<int32_t>();
+      break;
+    case 1:
+      n.kind = NodeKind::Sum;
+      n.children = body.getList(0).toVector<int32_t>();
+      n.weights = body.getList(1).toVector<double>();
+      break;
+    case 2:
+      n.kind = NodeKind::Histogram;
+      n.breaks = body.getList(0).toVector<int32_t>();
+      n.densities = body.getList(1).toVector<double>();
+      n.scope = body.get<int32_t>(4);
+      break;
+    case 3:
+      n.kind = NodeKind::Gaussian;
+      n.mean = body.get<double>(0);
+      n.stddev = body.get<double>(8);
+      n.scope = body.get<int32_t>(16);
+      break;
+    case 4:
+      n.kind = NodeKind::Categorical;
+      n.probabilities = body.getList(0).toVector<double>();
+      n.scope = body.get<int32_t>(0);
+      break;
+    default:
+      fatal("Unsupported node type " + std::to_string(which));
+  }
+  return n;
+}
+
+RawModel decodeModel(const capnp::StructReader& m) {
+  RawModel out;
+  out.rootNode = m.get<int32_t>(0);
+  out.numFeatures = m.get<int32_t>(4);
+  out.name = m.getText(0);
+  out.featureType = m.getText(1);
+  out.scope = m.getList(2).toVector<int32_t>();
+  capnp::ListReader nodes = m.getList(3);
+  out.nodes.reserve(nodes.size());
+  for (size_t i = 0; i < nodes.size(); ++i) out.nodes.push_back(decodeNode(nodes.getStruct(i)));
+  return out;
+}
+
+}  // namespace
+
+RawQuery readQueryFile(const std::string& path) {
+  capnp::Message msg = capnp::Message::fromFile(path);
+  capnp::StructReader header = msg.root();
+  uint16_t which = header.get<uint16_t>(0);
+  if (which == 0) fatal("Cannot compile raw models");
+  if (which != 1) fatal("Unknown header content");
+  capnp::StructReader query = header.getStruct(0);
+  if (!query.hasPointer(0)) fatal("Can only deserialize joint queries");
+  RawQuery q;
+  q.batchSize = query.get<int32_t>(0);
+  q.errorKind = query.get<uint16_t>(4);
+  q.maxError = query.get<double>(8);
+  capnp::StructReader joint = query.getStruct(0);
+  if (!joint.hasPointer(0)) fatal("No model attached to query");
+  q.supportMarginal = joint.getBool(0);  // absent in files written before the field existed
+  q.model = decodeModel(joint.getStruct(0));
+  return q;
+}
+
+FeatureTypeInfo parseFeatureType(const std::string& text) {
+  // Accepts the spellings of the reference's translateTypeString
+  // (SPFlowToMLIRDeserializer.cpp:226-248): "[u]int<width>" and "float<width>".
+  auto digits = [](const std::string& s, size_t from) -> int {
+    if (from >= s.size()) return -1;
+    int v = 0;
+    for (size_t i = from; i < s.size(); ++i) {
+      if (s[i] < '1' || s[i] > '9') return -1;
+      v = v * 10 + (s[i] - '0');
+      if (v > 4096) return -1;
+    }
+    return v;
+  };
+  size_t p = 0;
+  if (text.rfind("uint", 0) == 0) p = 4;
+  else if (text.rfind("int", 0) == 0) p = 3;
+  if (p) {
+    switch (digits(text, p)) {
+      case 8: return {FeatureType::U8, 1, false, "unsigned char"};
+      case 16: return {FeatureType::U16, 2, false, "unsigned short"};
+      case 32: return {FeatureType::U32, 4, false, "unsigned int"};
+      case 64: return {FeatureType::U64, 8, false, "unsigned long long"};
+      default: fatal("Unsupported feature data type " + text);
+    }
+  }
+  if (text.rfind("float", 0) == 0) {
+    switch (digits(text, 5)) {
+      case 32: return {FeatureType::F32, 4, true, "float"};
+      case 64: return {FeatureType::F64, 8, true, "double"};
+      case -1: break;
+      default: fatal("Unsupported floating-point type " + text);
+    }
+  }
+  fatal("Unsupported feature data type " + text);
+}
+
+namespace {
+
+void checkNormalized(const std::vector<double>& v, const char* msg) {
+  double sum = 0;
+  for (double p : v) sum += p;
+  if (!(std::fabs(sum - 1.0) <= 1e-6)) fatal(msg);
+}
+
+// Flat [0, maxUB) density table with zeros in gaps; the same table the reference builds before
+// taking logs (mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:447-493).
+std::vector<double> histogramTable(const RawNode& n) {
+  if (n.breaks.size() < 2) fatal("Histogram needs at least two breaks");
+  size_t buckets = n.breaks.size() - 1;
+  if (n.densities.size() < buckets) fatal("bucketCount must match the actual number of buckets!");
+  std::vector<std::pair<int64_t, int64_t>> iv;
+  int64_t minLB = INT64_MAX, maxUB = INT64_MIN;
+  for (size_t i = 0; i < buckets; ++i) {
+    int64_t lb = n.breaks[i], ub = n.breaks[i + 1];
+    if (ub < lb) fatal("Lower bound must be less or equal to upper bound!");
+    iv.emplace_back(lb, ub);
+    minLB = std::min(minLB, lb);
+    maxUB = std::max(maxUB, ub);
+  }
+  std::vector<std::pair<int64_t, int64_t>> sorted = iv;
+  std::sort(sorted.begin(), sorted.end());
+  for (size_t i = 1; i < sorted.size(); ++i)
+    if (sorted[i].first < sorted[i - 1].second) fatal("Overlapping buckets in histogram!");
+  if (minLB < 0) fatal("Histogram buckets with negative lower bound are not supported");
+  if (maxUB > (int64_t(1) << 24)) fatal("Histogram upper bound too large");
+  std::vector<double> tab(size_t(maxUB), 0.0);
+  for (size_t i = 0; i < buckets; ++i)
+    for (int64_t v = iv[i].first; v < iv[i].second; ++v) tab[size_t(v)] = n.densities[i];
+  return tab;
+}
+
+void appendBytes(std::string& key, const void* p, size_t n) { key.append(reinterpret_cast<const char*>(p), n); }
+
+std::string structuralKey(const GraphNode& g) {
+  std::string key;
+  key.push_back(char(g.kind));
+  switch (g.kind) {
+    case NodeKind::Gaussian:
+      appendBytes(key, &g.feature, 4);
+      appendBytes(key, &g.mean, 8);
+      appendBytes(key, &g.stddev, 8);
+      break;
+    case NodeKind::Categorical:
+    case NodeKind::Histogram:
+      appendBytes(key, &g.feature, 4);
+      appendBytes(key, g.table.data(), g.table.size() * 8);
+      break;
+    case NodeKind::Sum:
+      appendBytes(key, g.weights.data(), g.weights.size() * 8);
+      [[fallthrough]];
+    case NodeKind::Product:
+      appendBytes(key, g.children.data(), g.children.size() * 4);
+      break;
+  }
+  return key;
+}
+
+}  // namespace
+
+Graph buildGraph(const RawQuery& q) {
+  const RawModel& m = q.model;
+  Graph g;
+  g.name = m.name.empty() ? std::string("spn_kernel") : m.name;
+  g.ftype = parseFeatureType(m.featureType);
+  g.supportMarginal = q.supportMarginal;
+  g.batchSize = q.batchSize;
+  if (m.numFeatures <= 0) fatal("Query has no input features");
+  if (size_t(m.numFeatures) != m.scope.size()) fatal("Number of features does not match the size of the scope");
+  g.numFeatures = uint32_t(m.numFeatures);
+  if (q.supportMarginal && !g.ftype.isFloat) fatal("Feature data type must be floating-point to support marginal");
+
+  // Scope values map to input columns in ascending order.
+  std::vector<int32_t> sortedScope = m.scope;
+  std::sort(sortedScope.begin(), sortedScope.end());
+  std::map<int32_t, uint32_t> column;
+  for (size_t i = 0; i < sortedScope.size(); ++i) column[sortedScope[i]] = uint32_t(i);
+
+  // Pass 1: validate every serialized node in file order; children must already be defined.
+  std::unordered_map<int32_t, size_t> defined;  // id -> index into m.nodes
+  for (size_t i = 0; i < m.nodes.size(); ++i) {
+    const RawNode& n = m.nodes[i];
+    switch (n.kind) {
+      case NodeKind::Product:
+        if (n.children.empty()) fatal("Number of operands must be at least one");
+        break;
+      case NodeKind::Sum:
+        if (n.weights.size() != n.children.size()) fatal("Number of weights must match the number of addends!");
+        if (n.children.empty()) fatal("Number of addends must be greater than zero!");
+        checkNormalized(n.weights, "Weights must sum up to 1.0 for normalized SPN");
+        break;
+      case NodeKind::Categorical:
+        checkNormalized(n.probabilities, "Category probabilities should sum to 1.0");
+        [[fallthrough]];
+      case NodeKind::Histogram:
+      case NodeKind::Gaussian:
+        if (!column.count(n.scope)) fatal("Leaf node references unknown feature!");
+        break;
+    }
+    for (int32_t c : n.children)
+      if (!defined.count(c)) fatal("No definition found for node with ID: " + std::to_string(c));
+    defined[n.id] = i;
+  }
+  if (!defined.count(m.rootNode)) fatal("No definition found for node with ID: " + std::to_string(m.rootNode));
+  g.stats.serializedNodes = uint32_t(m.nodes.size());
+
+  // Pass 2: depth-first post-order from the root with structural deduplication.
+  std::unordered_map<size_t, uint32_t> placed;         // raw index -> graph index
+  std::unordered_map<std::string, uint32_t> interned;  // structural key -> graph index
+  struct Frame {
+    size_t raw;
+    size_t next;
+  };
+  std::vector<Frame> stack{{defined[m.rootNode], 0}};
+  while (!stack.empty()) {
+    Frame& f = stack.back();
+    const RawNode& n = m.nodes[f.raw];
+    if (placed.count(f.raw)) {
+      stack.pop_back();
+      continue;
+    }
+    if (f.next < n.children.size()) {
+      size_t child = defined[n.children[f.next++]];
+      if (!placed.count(child)) stack.push_back({child, 0});
+      continue;
+    }
+    GraphNode gn;
+    gn.kind = n.kind;
+    switch (n.kind) {
+      case NodeKind::Product:
+      case NodeKind::Sum:
+        for (int32_t c : n.children) gn.children.push_back(placed.at(defined[c]));
+        gn.weights = n.weights;
+        break;
+      case NodeKind::Gaussian:
+        gn.feature = column[n.scope];
+        gn.mean = n.mean;
+        gn.stddev = n.stddev;
+        if (!(n.stddev > 0) || !std::isfinite(n.stddev) || !std::isfinite(n.mean))
+          fatal("Gaussian leaf needs a finite mean and a positive finite standard deviation");
+        break;
+      case NodeKind::Categorical:
+        gn.feature = column[n.scope];
+        gn.table = n.probabilities;
+        break;
+      case NodeKind::Histogram:
+        gn.feature = column[n.scope];
+        gn.table = histogramTable(n);
+        break;
+    }
+    std::string key = structuralKey(gn);
+    auto it = interned.find(key);
+    uint32_t idx;
+    if (it != interned.end()) {
+      idx = it->second;
+    } else {
+      idx = uint32_t(g.nodes.size());
+      g.nodes.push_back(std::move(gn));
+      interned.emplace(std::move(key), idx);
+    }
+    placed[f.raw] = idx;
+    stack.pop_back();
+  }
+  // The root must be the last node; with deduplication it always is, because nothing is
+  // appended after the root is placed.
+  uint32_t rootIdx = placed.at(defined[m.rootNode]);
+  if (rootIdx != g.nodes.size() - 1) fatal("internal error: root is not last in schedule");
+
+  // Use counts and statistics.
+  for (auto& n : g.nodes)
+    for (uint32_t c : n.children) g.nodes[c].uses++;
+  g.nodes.back().uses++;
+  GraphStats& st = g.stats;
+  uint64_t leafSelect = q.supportMarginal ? 1 : 0;
+  for (const auto& n : g.nodes) {
+    uint64_t k = n.children.size();
+    st.maxFanIn = std::max<uint32_t>(st.maxFanIn, uint32_t(k));
+    switch (n.kind) {
+      case NodeKind::Gaussian:
+        st.gaussians++;
+        st.flopsMin += 4 + leafSelect;
+        st.flopsPairwise += 4 + leafSelect;
+        break;
+      case NodeKind::Categorical:
+        st.categoricals++;
+        st.flopsMin += leafSelect;
+        st.flopsPairwise += leafSelect;
+        break;
+      case NodeKind::Histogram:
+        st.histograms++;
+        st.flopsMin += leafSelect;
+        st.flopsPairwise += leafSelect;
+        break;
+      case NodeKind::Product:
+        st.products++;
+        st.productAdds += k - 1;
+        st.flopsMin += k - 1;
+        st.flopsPairwise += k - 1;
+        break;
+      case NodeKind::Sum: {
+        st.sums++;
+        st.sumTerms += k;
+        uint64_t fp = 8 * k - 7, tp = 2 * (k - 1);
+        uint64_t fn = 5 * k, tn = k + 1;
+        st.flopsPairwise += fp;
+        st.transPairwise += tp;
+        if (k <= 1) {
+          st.flopsMin += 1;  // a single weighted child is one add
+        } else if (fp + 3 * tp <= fn + 3 * tn) {
+          st.flopsMin += fp;
+          st.transMin += tp;
+        } else {
+          st.flopsMin += fn;
+          st.transMin += tn;
+        }
+        break;
+      }
+    }
+  }
+  return g;
+}
+
+}  // namespace spnc_hip

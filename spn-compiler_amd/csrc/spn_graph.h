@@ -1,0 +1,103 @@
+// SPN query model: what the reader produces from a serialized query, and the validated,
+// deduplicated, topologically scheduled DAG the kernel generators consume.
+//
+// Semantics follow the reference frontend
+// (compiler/src/pipeline/steps/frontend/SPFlowToMLIRDeserializer.cpp:63-248) and the HiSPN
+// verifiers (mlir/lib/Dialect/HiSPN/HiSPNOps.cpp:31-125).
+#pragma once
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace spnc_hip {
+
+enum class NodeKind : uint8_t { Product = 0, Sum = 1, Histogram = 2, Gaussian = 3, Categorical = 4 };
+
+// A node exactly as serialized (ids, scope values).
+struct RawNode {
+  int32_t id = 0;
+  NodeKind kind = NodeKind::Product;
+  bool root = false;
+  std::vector<int32_t> children;
+  std::vector<double> weights;
+  int32_t scope = -1;
+  double mean = 0, stddev = 1;
+  std::vector<double> probabilities;
+  std::vector<int32_t> breaks;
+  std::vector<double> densities;
+};
+
+struct RawModel {
+  int32_t rootNode = 0;
+  int32_t numFeatures = 0;
+  std::string name, featureType;
+  std::vector<int32_t> scope;
+  std::vector<RawNode> nodes;
+};
+
+struct RawQuery {
+  int32_t batchSize = 1;
+  uint16_t errorKind = 0;
+  double maxError = 0;
+  bool supportMarginal = false;
+  RawModel model;
+};
+
+// Reads a serialized query. Throws std::runtime_error with the reference's messages for raw
+// models ("Cannot compile raw models"), queries without a joint ("Can only deserialize joint
+// queries") and joints without a model ("No model attached to query").
+RawQuery readQueryFile(const std::string& path);
+
+enum class FeatureType : uint8_t { U8, U16, U32, U64, F32, F64 };
+
+struct FeatureTypeInfo {
+  FeatureType type;
+  unsigned bytes;
+  bool isFloat;
+  const char* hipName;  // spelling of the type in generated device code
+};
+// Parses "[u]int<W>" / "float<W>"; integers are treated as unsigned of that width, as the
+// reference does (uitofp / index_cast). Throws "Unsupported feature data type <text>".
+FeatureTypeInfo parseFeatureType(const std::string& text);
+
+// A DAG node after validation: children are indices into Graph::nodes (always smaller than
+// the node's own index), leaves carry the input column and a flat linear-space table.
+struct GraphNode {
+  NodeKind kind;
+  uint32_t feature = 0;            // input column (leaves)
+  std::vector<uint32_t> children;  // inner nodes
+  std::vector<double> weights;     // sums, linear space
+  double mean = 0, stddev = 1;     // Gaussian
+  std::vector<double> table;       // Categorical: probabilities; Histogram: flat [0,maxUB) densities, 0 in gaps
+  uint32_t uses = 0;               // number of parents (root counts as one use)
+};
+
+struct GraphStats {
+  uint32_t gaussians = 0, categoricals = 0, histograms = 0, products = 0, sums = 0;
+  uint64_t productAdds = 0;   // sum over products of (k-1)
+  uint64_t sumTerms = 0;      // sum over sums of k
+  uint32_t maxFanIn = 0;
+  uint32_t serializedNodes = 0;  // before dropping unreachable nodes and merging duplicates
+  // Algorithmic work per sample: cheaper of pairwise tree (k==2) and n-ary LSE (k>=3) per sum,
+  // 4 flops per Gaussian, 0 per table leaf, +1 select per leaf when marginal.
+  uint64_t flopsMin = 0, transMin = 0, flopsPairwise = 0, transPairwise = 0;
+  uint64_t issueSlotsMin() const { return flopsMin + 3 * transMin; }
+};
+
+struct Graph {
+  std::string name;
+  FeatureTypeInfo ftype;
+  uint32_t numFeatures = 0;
+  bool supportMarginal = false;
+  int32_t batchSize = 1;
+  std::vector<GraphNode> nodes;  // children first; root is nodes.back()
+  GraphStats stats;
+  uint32_t root() const { return uint32_t(nodes.size() - 1); }
+};
+
+// Validates the query and builds the scheduled DAG: only nodes reachable from the root,
+// depth-first post-order (children first, left to right), structurally identical nodes merged.
+// Throws std::runtime_error on every rule the reference rejects.
+Graph buildGraph(const RawQuery& q);
+
+}  // namespace spnc_hip
