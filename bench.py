@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the batched joint log-likelihood path on one MI355X.
+
+A step is one pass of the compiled SPN kernel over one batch of synthetic inputs that already
+sit in HBM. The headline workload is configuration C2 (random sum/product tree over 16 Gaussian
+features, 16M float32 rows); ``--config`` selects another one, and the remaining configurations
+are measured with a few steps each and reported under "others" in the same JSON line.
+
+Prints ONE JSON line: samples/s, the roofline of the kernel (HIP-event timed launches) and a CPU
+baseline (the restated CPUCompiler-equivalent kernel of oracle/cgen.py on the host cores).
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "spn-compiler_amd"))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X FP32 vector, published
+
+
+def make_inputs(name, cfg, n, torch, device):
+    """Synthetic inputs of the configuration's shape and distribution, generated on the device."""
+    from spnc import synthetic as syn
+    g = torch.Generator(device=device)
+    g.manual_seed({"c1": 1, "c2": 102, "c3": 103, "c4": 104, "c5": 102}[name])
+    F = cfg["features"]
+    if name == "c1":
+        return torch.randint(0, 3, (n, F), generator=g, device=device, dtype=torch.int32)
+    if name == "c3":
+        doms = torch.tensor([d for _, d in syn.c3_domains()], device=device, dtype=torch.float32)
+        u = torch.rand((n, F), generator=g, device=device)
+        return torch.minimum((u * doms).floor(), doms - 1).to(torch.int32)
+    x = torch.randn((n, F), generator=g, device=device, dtype=torch.float32)
+    if name == "c5":
+        g2 = torch.Generator(device=device)
+        g2.manual_seed(105)
+        mask = torch.rand((n, F), generator=g2, device=device) < 0.2
+        x[mask] = float("nan")
+    return x
+
+
+def measure(name, n, steps, warmup, torch, device, extra_options=None):
+    from spnc import synthetic as syn
+    from spnc.hip import HIPCompiler
+    cfg = syn.CONFIGS[name]
+    n = n or cfg["n"]
+    spn = cfg["spn"]()
+    t0 = time.time()
+    kernel = HIPCompiler(**(extra_options or {})).compile_ll(spn, cfg["dtype"], supportMarginal=cfg["marginal"])
+    compile_s = time.time() - t0
+    info = kernel.info()
+    x = make_inputs(name, cfg, n, torch, device)
+    out = torch.empty(n, device=device, dtype=torch.float32 if info["dtype"] == "float32" else torch.float64)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        kernel.execute_device(n, x.data_ptr(), out.data_ptr(), stream)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    launch_ms = sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
+    finite = bool(torch.isfinite(out[: min(n, 1 << 20)]).all().item())
+
+    bytes_per_sample = cfg["features"] * info["bytes_per_feature"] + info["bytes_per_result"]
+    flops, trans = info["flops_min"], info["trans_min"]
+    slots = flops + 3 * trans
+    props = torch.cuda.get_device_properties(device)
+    clock_hz = props.clock_rate * 1e3 if hasattr(props, "clock_rate") else 2.4e9
+    valu_peak = props.multi_processor_count * 64 * clock_hz  # lane-operations per second
+    t_launch = launch_ms * 1e-3
+    hbm_gbs = bytes_per_sample * n / t_launch / 1e9
+    tflops = flops * n / t_launch / 1e12
+    t_min_hbm = bytes_per_sample * n / (HBM_PEAK_GBS * 1e9)
+    t_min_valu = slots * n / valu_peak
+    hbm_bound = t_min_hbm >= t_min_valu
+    roof = {
+        "bound": "hbm" if hbm_bound else "valu-fp32",
+        "achieved": round(hbm_gbs if hbm_bound else tflops, 3),
+        "peak": HBM_PEAK_GBS if hbm_bound else FP32_VECTOR_PEAK_TFLOPS,
+        "unit": "GB/s" if hbm_bound else "TFLOP/s",
+        "frac": round((hbm_gbs / HBM_PEAK_GBS) if hbm_bound else (tflops / FP32_VECTOR_PEAK_TFLOPS), 4),
+        "traffic": None,
+        "kernel": "spn_kernel (hipRTC straight-line)" if info["kernel_kind"] == 1 else "spn_interp_kernel",
+        "launch_ms": round(launch_ms, 4),
+        "bytes_per_sample": bytes_per_sample,
+        "flops_per_sample": flops,
+        "transcendentals_per_sample": trans,
+        "issue_slots_per_sample": slots,
+        "valu_issue_peak_per_s": valu_peak,
+        "valu_issue_frac": round(t_min_valu / t_launch, 4),
+        "hbm_frac": round(t_min_hbm / t_launch, 4),
+    }
+    res = {
+        "workload": name, "desc": cfg["desc"], "n": n, "samples_per_s": n * steps / wall, "ms_per_step": wall / steps * 1e3,
+        "roofline": roof, "compile_s": round(compile_s, 2), "nodes": info["num_nodes"], "finite": finite,
+    }
+    os.remove(kernel.fileName())
+    return res, x, cfg, spn
+
+
+def cpu_baseline(name, cfg, spn, x_dev, torch):
+    """The restated CPUCompiler-equivalent kernel (oracle/cgen.py), timed on this host on a bounded
+    sample of the same inputs."""
+    sys.path.insert(0, ROOT)
+    from oracle import cgen, spn_model as sm
+    from xspn.serialization.binary.BinarySerialization import BinarySerializer
+    from xspn.structure.Model import SPNModel
+    from xspn.structure.Query import JointProbability
+    import contextlib
+    import io
+    with tempfile.TemporaryDirectory() as td:
+        path = os.path.join(td, "q.bin")
+        with contextlib.redirect_stdout(io.StringIO()):
+            BinarySerializer(path).serialize_to_file(JointProbability(SPNModel(spn, cfg["dtype"], "cpu"), batchSize=4096,
+                                                                      supportMarginal=cfg["marginal"]))
+        model = sm.load_model(path)
+        so, _ = cgen.build(model, cfg["marginal"], workdir=td)
+        run = cgen.load(so, cfg["dtype"])
+        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+        probe_n = min(x_dev.shape[0], 1 << 16)
+        xp = x_dev[:probe_n].cpu().numpy()
+        run(xp[:4096])
+        t0 = time.perf_counter()
+        run(xp)
+        rate = probe_n / (time.perf_counter() - t0)
+        sample_n = int(min(x_dev.shape[0], max(probe_n, rate * 5.0)))  # about 5 s per pass
+        xs = x_dev[:sample_n].cpu().numpy()
+        best = 0.0
+        t_all = time.perf_counter()
+        for _ in range(3):
+            t0 = time.perf_counter()
+            run(xs)
+            best = max(best, sample_n / (time.perf_counter() - t0))
+            if time.perf_counter() - t_all > 20:
+                break
+    return {"value": best, "unit": "samples/s", "cores": cores, "kind": "port",
+            "sample": f"first {sample_n} rows of the same batch, best of up to 3 passes, gcc -O3 -march=native + OpenMP chunks of 4096"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--n", type=int, default=0, help="override the number of samples")
+    ap.add_argument("--no-others", action="store_true", help="measure only the selected configuration")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--opt", action="append", default=[], help="extra compiler option key=value")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: samples are independent, a multi-GPU run would only split the batch; use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import contextlib
+    import io
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    extra = dict(kv.split("=", 1) for kv in args.opt)
+    log = io.StringIO()
+    with contextlib.redirect_stdout(log):
+        res, x, cfg, spn = measure(args.config, args.n, args.steps, args.warmup, torch, device, extra)
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(args.config, cfg, spn, x, torch)
+    del x
+    torch.cuda.empty_cache()
+    others = {}
+    if not args.no_others:
+        for name in ["c1", "c2", "c3", "c4", "c5"]:
+            if name == args.config:
+                continue
+            with contextlib.redirect_stdout(log):
+                r, xo, _, _ = measure(name, 0, max(3, args.steps // 4), 2, torch, device, extra)
+            del xo
+            torch.cuda.empty_cache()
+            others[name] = {"samples_per_s": round(r["samples_per_s"], 1), "n": r["n"], "ms_per_step": round(r["ms_per_step"], 4),
+                            "roofline": r["roofline"], "nodes": r["nodes"]}
+    line = {
+        "metric": "samples/sec log-likelihood on 1 MI355X + % of HBM/FP32 roofline",
+        "value": round(res["samples_per_s"], 1),
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(res["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic (seeded, generated on the device; random SPN parameters from seeded NumPy generators)",
+        "config": {"workload": f"{args.config}: {res['desc']}", "samples": res["n"], "nodes": res["nodes"]},
+        "roofline": res["roofline"],
+        "cpu_baseline": cpu,
+        "others": others,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,9 +1,11 @@
 #include "emit_hip.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <sstream>
 #include <stdexcept>
+#include <vector>
 
 namespace spnc_hip {
 
@@ -23,6 +25,7 @@ struct Emitter {
   std::vector<bool> featGauss;         // per feature: used by a Gaussian leaf
   std::vector<bool> featUsed;
   std::vector<bool> featPrepared;
+  std::vector<bool> emitted;
   bool vectorRows = true;
 
   Emitter(const Graph& graph, const CompileOptions& opts) : g(graph), o(opts) {
@@ -72,6 +75,7 @@ struct Emitter {
     featGauss.assign(g.numFeatures, false);
     featUsed.assign(g.numFeatures, false);
     featPrepared.assign(g.numFeatures, false);
+    emitted.assign(g.nodes.size(), false);
     for (const auto& n : g.nodes) {
       if (n.kind == NodeKind::Gaussian) {
         featGauss[n.feature] = true;
@@ -126,14 +130,11 @@ struct Emitter {
     }
   }
 
-  std::string expOf(const std::string& a) const {
-    if (f64) return "exp(" + a + ")";
-    return log2Dom ? "__builtin_amdgcn_exp2f(" + a + ")" : "expf(" + a + ")";
-  }
-  std::string logOf(const std::string& a) const {
-    if (f64) return "log(" + a + ")";
-    return log2Dom ? "__builtin_amdgcn_logf(" + a + ")" : "logf(" + a + ")";
-  }
+  // The log2-domain f32 kernel uses the hardware exp2/log2 instructions directly. The other
+  // flavours call the accurate library routines through out-of-line wrappers: inlining them
+  // thousands of times into one basic block makes register allocation take minutes.
+  std::string expOf(const std::string& a) const { return (log2Dom ? "__builtin_amdgcn_exp2f(" : "spn_exp(") + a + ")"; }
+  std::string logOf(const std::string& a) const { return (log2Dom ? "__builtin_amdgcn_logf(" : "spn_log(") + a + ")"; }
   std::string maxOf(const std::string& a, const std::string& b) const {
     return std::string(f64 ? "__builtin_fmax(" : "__builtin_fmaxf(") + a + ", " + b + ")";
   }
@@ -149,7 +150,11 @@ struct Emitter {
     }
   }
 
+  // Emits node i after everything it depends on. Children are emitted lazily, right before
+  // their first use, so that a sum over hundreds of children never holds all of them live.
   void emitNode(uint32_t i) {
+    if (emitted[i]) return;
+    emitted[i] = true;
     const auto& n = g.nodes[i];
     if (n.kind != NodeKind::Product && n.kind != NodeKind::Sum) emitFeaturePrep(n.feature);
     switch (n.kind) {
@@ -165,7 +170,7 @@ struct Emitter {
           emitLeafMarginal(i, lit(coef * scale) + " + (" + d + " * " + d + ") * " + lit(den * scale));
         } else {
           double coef = 1.0 / std::sqrt(2.0 * M_PI * n.stddev * n.stddev);
-          emitLeafMarginal(i, lit(coef) + " * exp((" + d + " * " + d + ") * " + lit(den) + ")");
+          emitLeafMarginal(i, lit(coef) + " * spn_exp((" + d + " * " + d + ") * " + lit(den) + ")");
         }
         break;
       }
@@ -176,7 +181,11 @@ struct Emitter {
       case NodeKind::Product: {
         const char* op = logSpace ? " + " : " * ";
         std::string e = tree(
-            0, n.children.size(), [&](size_t k) { return v(n.children[k]); },
+            0, n.children.size(),
+            [&](size_t k) {
+              emitNode(n.children[k]);
+              return v(n.children[k]);
+            },
             [&](const std::string& a, const std::string& b) { return "(" + a + op + b + ")"; });
         body << "  const real_t " << v(i) << " = " << e << ";\n";
         break;
@@ -189,56 +198,71 @@ struct Emitter {
 
   void emitSum(uint32_t i) {
     const auto& n = g.nodes[i];
-    size_t k = n.children.size();
+    const size_t k = n.children.size();
+    std::string p = "s" + std::to_string(i) + "_";
+    unsigned tmp = 0;
+    auto fresh = [&](const std::string& expr) {
+      std::string name = p + "t" + std::to_string(tmp++);
+      body << "  const real_t " << name << " = " << expr << ";\n";
+      return name;
+    };
     if (!logSpace) {
+      // Linear space: child * weight, then the balanced tree of adds; partial sums are named so
+      // that the expression stays flat for sums with hundreds of children.
       std::string e = tree(
-          0, k, [&](size_t j) { return "(" + v(n.children[j]) + " * " + lit(n.weights[j]) + ")"; },
-          [&](const std::string& a, const std::string& b) { return "(" + a + " + " + b + ")"; });
+          0, k,
+          [&](size_t j) {
+            emitNode(n.children[j]);
+            return fresh(v(n.children[j]) + " * " + lit(n.weights[j]));
+          },
+          [&](const std::string& a, const std::string& b) { return fresh(a + " + " + b); });
       body << "  const real_t " << v(i) << " = " << e << ";\n";
       return;
     }
-    auto term = [&](size_t j) { return "(" + v(n.children[j]) + " + " + lit(logConst(n.weights[j])) + ")"; };
+    auto term = [&](size_t j) {
+      emitNode(n.children[j]);
+      return fresh(v(n.children[j]) + " + " + lit(logConst(n.weights[j])));
+    };
     if (k == 1) {
       body << "  const real_t " << v(i) << " = " << term(0) << ";\n";
       return;
     }
-    std::string p = "s" + std::to_string(i) + "_";
     if (o.sumForm == SumForm::Pairwise) {
       // a + log1p(exp(b - a)) with a the larger operand, over the reference's balanced tree
       // (mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:216-240).
-      unsigned tmp = 0;
-      std::string e = tree(
-          0, k,
-          [&](size_t j) {
-            std::string name = p + "y" + std::to_string(j);
-            body << "  const real_t " << name << " = " << term(j) << ";\n";
-            return name;
-          },
-          [&](const std::string& a, const std::string& b) {
-            std::string name = p + "t" + std::to_string(tmp++);
-            body << "  const real_t " << name << " = spn_logadd(" << a << ", " << b << ");\n";
-            return name;
-          });
+      std::string e = tree(0, k, term, [&](const std::string& a, const std::string& b) { return fresh("spn_logadd(" + a + ", " + b + ")"); });
       body << "  const real_t " << v(i) << " = " << e << ";\n";
       return;
     }
-    // n-ary max-shifted log-sum-exp: m = max_j y_j, m + log(sum_j exp(y_j - m)).
-    for (size_t j = 0; j < k; ++j) body << "  const real_t " << p << "y" << j << " = " << term(j) << ";\n";
+    const std::string lowest = f64 ? "(-0x1.fffffffffffffp+1023)" : "(-0x1.fffffep+127f)";
     if (k == 2) {
-      // log(1 + exp(-|y0 - y1|)): the larger term contributes exp(0) = 1 exactly.
+      // max + log(1 + exp(-|y0 - y1|)): the larger term contributes exp(0) = 1 exactly. Two
+      // impossible children give exp(NaN); the max with 0 turns that into log(1 + 0).
+      std::string y0 = term(0), y1 = term(1);
       std::string absf = f64 ? "__builtin_fabs" : "__builtin_fabsf";
-      body << "  const real_t " << v(i) << " = " << maxOf(p + "y0", p + "y1") << " + "
-           << logOf(lit(1.0) + " + " + expOf("-" + absf + "(" + p + "y0 - " + p + "y1)")) << ";\n";
+      body << "  const real_t " << v(i) << " = " << maxOf(y0, y1) << " + "
+           << logOf(lit(1.0) + " + " + maxOf(expOf("-" + absf + "(" + y0 + " - " + y1 + ")"), lit(0.0))) << ";\n";
       return;
     }
-    std::string m = tree(
-        0, k, [&](size_t j) { return p + "y" + std::to_string(j); },
-        [&](const std::string& a, const std::string& b) { return maxOf(a, b); });
-    body << "  const real_t " << p << "m = " << m << ";\n";
-    std::string s = tree(
-        0, k, [&](size_t j) { return expOf(p + "y" + std::to_string(j) + " - " + p + "m"); },
-        [&](const std::string& a, const std::string& b) { return "(" + a + " + " + b + ")"; });
-    body << "  const real_t " << v(i) << " = " << p << "m + " << logOf(s) << ";\n";
+    // n-ary max-shifted log-sum-exp, m + log(sum_j exp(y_j - m)) with m = max_j y_j, evaluated
+    // over chunks of children with a running (m, s): s <- s * exp(m_old - m_new) + sum_chunk exp(y_j - m_new).
+    // m is clamped to the lowest finite value so that impossible children (-inf) give exp(-inf) = 0, not NaN.
+    const size_t chunk = 16;
+    std::string m, sAcc;
+    for (size_t lo = 0; lo < k; lo += chunk) {
+      const size_t hi = std::min(k, lo + chunk);
+      std::vector<std::string> y;
+      for (size_t j = lo; j < hi; ++j) y.push_back(term(j));
+      std::string cm = tree(
+          0, y.size(), [&](size_t j) { return y[j]; }, [&](const std::string& a, const std::string& b) { return maxOf(a, b); });
+      std::string mNew = fresh(maxOf(lo == 0 ? cm : maxOf(m, cm), lowest));
+      std::string part = tree(
+          0, y.size(), [&](size_t j) { return expOf(y[j] + " - " + mNew); },
+          [&](const std::string& a, const std::string& b) { return "(" + a + " + " + b + ")"; });
+      sAcc = lo == 0 ? fresh(part) : fresh(sAcc + " * " + expOf(m + " - " + mNew) + " + " + part);
+      m = mNew;
+    }
+    body << "  const real_t " << v(i) << " = " << m << " + " << logOf(sAcc) << ";\n";
   }
 };
 
@@ -259,7 +283,8 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   js.bytesPerResult = e.f64 ? 8 : 4;
   js.tableEntries = unsigned(e.tablePool.size());
   const unsigned realBytes = e.f64 ? 8 : 4;
-  js.tablesInLds = js.tableEntries > 0 && size_t(js.tableEntries) * realBytes <= 48 * 1024;
+  // gfx950 has 160 KiB of LDS per CU, all of it usable by one workgroup.
+  js.tablesInLds = js.tableEntries > 0 && size_t(js.tableEntries) * realBytes <= 140 * 1024;
 
   const unsigned F = g.numFeatures;
   const unsigned eb = g.ftype.bytes;
@@ -291,8 +316,12 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     for (size_t i = 0; i < e.tablePool.size(); ++i) s << (i ? ", " : "") << (i % 8 == 0 ? "\n  " : "") << e.lit(e.tablePool[i]);
     s << "};\n";
   }
+  if (!e.log2Dom) {
+    s << "static __device__ __attribute__((noinline)) real_t spn_exp(real_t x) { return " << (e.f64 ? "exp(x)" : "expf(x)") << "; }\n";
+    s << "static __device__ __attribute__((noinline)) real_t spn_log(real_t x) { return " << (e.f64 ? "log(x)" : "logf(x)") << "; }\n";
+  }
   if (e.logSpace && o.sumForm == SumForm::Pairwise) {
-    s << "static __device__ __forceinline__ real_t spn_logadd(real_t x, real_t y) {\n"
+    s << "static __device__ " << (e.log2Dom ? "__forceinline__" : "__attribute__((noinline))") << " real_t spn_logadd(real_t x, real_t y) {\n"
          "  const bool gt = x > y;\n  const real_t a = gt ? x : y;\n  const real_t b = gt ? y : x;\n";
     if (e.f64) s << "  return a + log1p(exp(b - a));\n";
     else if (e.log2Dom) s << "  return a + __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(b - a));\n";
@@ -320,14 +349,14 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     s << "}\n";
   }
 
-  for (uint32_t i = 0; i < g.nodes.size(); ++i) e.emitNode(i);
+  e.emitNode(g.root());
   if (e.vectorRows)
     s << "static __device__ __forceinline__ real_t spn_eval(const feat_t (&x)[SPN_F], const real_t* __restrict__ tab) {\n";
   else
     s << "static __device__ __forceinline__ real_t spn_eval(const feat_t* __restrict__ row, const real_t* __restrict__ tab) {\n";
   s << e.body.str();
   std::string root = Emitter::v(g.root());
-  if (!e.logSpace) s << "  return log(" << root << ");\n";
+  if (!e.logSpace) s << "  return spn_log(" << root << ");\n";
   else if (e.log2Dom) s << "  return " << root << " * 0x1.62e43p-1f;\n";  // back to natural log: * ln 2
   else s << "  return " << root << ";\n";
   s << "}\n";

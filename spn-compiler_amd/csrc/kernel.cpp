@@ -130,7 +130,11 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
   k->stats_ = g.stats;
   k->numNodes_ = unsigned(g.nodes.size());
 
-  const uint64_t ops = g.nodes.size() + g.stats.sumTerms + g.stats.productAdds;
+  // Size estimate that decides between the two kernels under "auto": terms of sums weigh more
+  // when the kernel calls the accurate library exp/log (float64 and natural-log float32) than
+  // when it uses the hardware exp2/log2 instructions.
+  const bool hardwareTranscendentals = o.useLogSpace && o.computeType == ComputeType::F32 && o.log2Domain;
+  const uint64_t ops = g.nodes.size() + g.stats.productAdds + g.stats.sumTerms * (hardwareTranscendentals ? 1 : 6);
   bool useInterp = o.kernelMode == KernelMode::Interpreter || (o.kernelMode == KernelMode::Auto && ops > uint64_t(std::max(0, o.jitMaxOps)));
   if (useInterp && !o.useLogSpace) {
     if (o.kernelMode == KernelMode::Interpreter) fatal("COMPILATION ERROR: the interpreter kernel supports log-space computation only");

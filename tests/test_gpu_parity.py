@@ -1,0 +1,316 @@
+"""Parity of the HIP kernels with the CPU oracle, through the C-ABI, on a real MI355X.
+
+Tolerances: |delta| <= 1e-4 absolute log-likelihood for f32 kernels, <= 1e-10 for f64 kernels
+(the bars the path is specified to), checked against the oracle's restatement of the reference's
+CPU kernel (``ll_reforder``) and against the float64 closed form.
+"""
+import math
+import os
+
+import numpy as np
+import pytest
+
+import rawfile as rf
+from conftest import GOLDEN, compile_query, compile_spn, load_golden, model_as_query, oracle_model, quiet
+from oracle import c_oracle, evaluate as ev, spn_model as sm
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-4
+F64_TOL = 1e-10
+
+VARIANTS = {
+    "jit": {},
+    "jit-pairwise": {"hip-sum-form": "pairwise"},
+    "jit-strict": {"hip-sum-form": "pairwise", "hip-log2-domain": "false"},
+    "interp": {"hip-kernel": "interpreter"},
+    "interp-natural": {"hip-kernel": "interpreter", "hip-log2-domain": "false"},
+}
+
+
+def run(kernel, X):
+    out = kernel.execute(X.shape[0], X)
+    os.remove(kernel.fileName()) if os.path.isfile(kernel.fileName()) else None
+    return out
+
+
+def check_f32(got, model, X, marginal):
+    assert got.dtype == np.float32 and got.shape == (X.shape[0],)
+    ref32 = ev.ll_reforder(model, X, np.float32, marginal=marginal)
+    ref64 = ev.ll_closed_f64(model, X, marginal=marginal)
+    finite = np.isfinite(ref64)
+    assert np.array_equal(np.isneginf(got), np.isneginf(ref64))
+    assert np.abs(got[finite] - ref64[finite]).max(initial=0) <= F32_TOL
+    ok = finite & np.isfinite(ref32)
+    assert np.abs(got[ok] - ref32[ok]).max(initial=0) <= F32_TOL
+
+
+# ---- the reference's own CUDA test cases (python-interface/test/cuda/*.py), run through HIPCompiler ----
+
+def _reference_test_spns():
+    from spnc import synthetic as syn
+    from spnc.structure import Gaussian, Histogram, Product, Sum
+    cat = syn.c1_spn()
+    gauss = Product(children=[Gaussian(mean=m, stdev=s, scope=i) for i, (m, s) in enumerate(
+        [(0.5, 1.0), (0.125, 0.25), (0.345, 0.24), (0.456, 0.1), (0.94, 0.48), (0.56, 0.42), (0.76, 0.14), (0.32, 0.58), (0.58, 0.219),
+         (0.14, 0.28)])])
+    h1 = Histogram([0., 1., 2.], [0.25, 0.75], [1, 1], scope=0)
+    h2 = Histogram([0., 1., 2.], [0.45, 0.55], [1, 1], scope=1)
+    h3 = Histogram([0., 1., 2.], [0.33, 0.67], [1, 1], scope=0)
+    h4 = Histogram([0., 1., 2.], [0.875, 0.125], [1, 1], scope=1)
+    hist = Sum(children=[Product(children=[h1, h2]), Product(children=[h3, h4])], weights=[0.3, 0.7])
+    return cat, gauss, hist
+
+
+@pytest.mark.parametrize("marginal", [False, True])
+def test_reference_cuda_test_cases(native, marginal):
+    from spnc.hip import HIPCompiler
+    rng = np.random.default_rng(7)
+    cat, gauss, hist = _reference_test_spns()
+    cases = [(cat, rng.integers(0, 3, (30, 6)).astype("float64")), (gauss, rng.normal(0.5, 1.0, (30, 10)).astype("float64")),
+             (hist, rng.integers(0, 2, (30, 2)).astype("float64"))]
+    for spn, X in cases:
+        if marginal:
+            X[rng.random(X.shape) < 0.3] = np.nan
+        for preload in (False, True):
+            with quiet():
+                got = HIPCompiler(preloadToSharedMem=preload).log_likelihood(spn, X, supportMarginal=marginal)
+            m = oracle_model(spn, "float64")
+            want = ev.ll_closed_f64(m, X, marginal=marginal)
+            # the reference's own acceptance criterion ...
+            assert np.all(np.isclose(got, want)) or np.all(np.isclose(np.exp(got), np.exp(want)))
+            # ... and the absolute bar of this path
+            check_f32(got, m, X, marginal)
+
+
+def test_integer_inputs_readme_example(native):
+    from spnc import synthetic as syn
+    from spnc.hip import HIPCompiler
+    X = syn.c1_inputs(30)
+    with quiet():
+        got = HIPCompiler().log_likelihood(syn.c1_spn(), X, supportMarginal=False)
+    check_f32(got, oracle_model(syn.c1_spn(), "int32"), X, False)
+
+
+@pytest.mark.parametrize("name", ["mini-example", "categorical-example", "gaussian-example"])
+def test_known_answers(native, name):
+    from test_oracle_pins import KNOWN
+    X, expected = KNOWN[name]
+    for opts in VARIANTS.values():
+        got = run(compile_query(native, os.path.join(GOLDEN, name + ".bin"), **opts), X)
+        assert np.allclose(got, expected, rtol=0, atol=6e-6)
+
+
+@pytest.mark.parametrize("variant", sorted(VARIANTS))
+@pytest.mark.parametrize("name", ["NIPS5", "nltcs", "plants"])
+def test_golden_outputs_f32(native, tmp_path, name, variant):
+    X, ref = load_golden(name)
+    if name == "NIPS5":
+        path, X = os.path.join(GOLDEN, "NIPS5.bin"), X.astype(np.uint32)
+    else:
+        path = model_as_query(os.path.join(GOLDEN, name + ".bin"), "float64", str(tmp_path / "q.bin"))
+    got = run(compile_query(native, path, **VARIANTS[variant]), X)
+    assert got.dtype == np.float32
+    assert np.abs(got - ref).max() <= F32_TOL
+
+
+@pytest.mark.parametrize("opts", [{"hip-compute-type": "float64"}, {"hip-compute-type": "float64", "hip-sum-form": "pairwise"},
+                                  {"hip-compute-type": "float64", "hip-kernel": "interpreter"}, {"use-log-space": "false"}],
+                         ids=["log-f64", "log-f64-pairwise", "log-f64-interp", "linear-f64"])
+@pytest.mark.parametrize("name", ["NIPS5", "nltcs", "plants"])
+def test_golden_outputs_f64(native, tmp_path, name, opts):
+    if name == "nltcs" and ("hip-sum-form" in opts or "use-log-space" in opts):
+        pytest.skip("float64 builds of the 3641-node model go to the interpreter; its straight-line float64 builds take minutes of hipRTC time")
+    X, ref = load_golden(name)
+    if name == "NIPS5":
+        path, X = os.path.join(GOLDEN, "NIPS5.bin"), X.astype(np.uint32)
+    else:
+        path = model_as_query(os.path.join(GOLDEN, name + ".bin"), "float64", str(tmp_path / "q.bin"))
+    got = run(compile_query(native, path, **opts), X)
+    assert got.dtype == np.float64
+    assert np.abs(got - ref).max() <= F64_TOL
+
+
+@pytest.mark.parametrize("variant", sorted(VARIANTS))
+@pytest.mark.parametrize("cfg", ["c1", "c2", "c3", "c4", "c5"])
+def test_benchmark_configurations(native, cfg, variant):
+    from spnc import synthetic as syn
+    c = syn.CONFIGS[cfg]
+    if cfg == "c4" and variant.startswith("jit-"):
+        pytest.skip("the 8881-node region graph is interpreter-sized; one straight-line build of it is enough")
+    n = 1500 if cfg == "c4" else 5000
+    spn, X = c["spn"](), c["inputs"](n)
+    got = run(compile_spn(native, spn, c["dtype"], marginal=c["marginal"], **VARIANTS[variant]), X)
+    m = oracle_model(spn, c["dtype"])
+    check_f32(got, m, X, c["marginal"])
+    assert np.abs(got - c_oracle.ll_f32(m, X, marginal=c["marginal"])).max() <= F32_TOL
+
+
+@pytest.mark.parametrize("kernel", ["jit", "interpreter"])
+def test_c5_marginal_in_f64(native, kernel):
+    from spnc import synthetic as syn
+    c = syn.CONFIGS["c5"]
+    spn, X = c["spn"](), c["inputs"](5000)
+    got = run(compile_spn(native, spn, "float32", marginal=True, **{"hip-compute-type": "float64", "hip-kernel": kernel}), X)
+    assert got.dtype == np.float64
+    m = oracle_model(spn, "float32")
+    assert np.abs(got - ev.ll_closed_f64(m, X, marginal=True)).max() <= F64_TOL
+    # linear-space float64 (the reference's own f64 kernel) on the same inputs
+    if kernel == "jit":
+        lin = run(compile_spn(native, spn, "float32", marginal=True, **{"use-log-space": "false"}), X)
+        assert np.abs(lin - ev.ll_linear_f64(m, X, marginal=True)).max() <= F64_TOL
+
+
+@pytest.mark.parametrize("dtype", ["uint8", "uint16", "int32", "uint32", "int64", "float32", "float64"])
+@pytest.mark.parametrize("kernel", ["jit", "interpreter"])
+def test_feature_types_and_out_of_range_inputs(native, dtype, kernel):
+    from spnc.structure import Categorical, Gaussian, Histogram, Product, Sum
+    spn = Sum(weights=[0.4, 0.6], children=[
+        Product(children=[Categorical(p=[0.2, 0.5, 0.3], scope=0), Gaussian(1.0, 2.0, scope=1),
+                          Histogram(breaks=[0, 2, 3, 6], densities=[0.1, 0.5, 0.1], bin_repr_points=[1, 2, 4], scope=2)]),
+        Product(children=[Categorical(p=[0.7, 0.3], scope=0), Gaussian(3.0, 1.5, scope=1),
+                          Histogram(breaks=[1, 4], densities=[1 / 3], bin_repr_points=[2], scope=2)])])
+    rng = np.random.default_rng(11)
+    X = np.column_stack([rng.integers(0, 5, 400), rng.integers(0, 7, 400), rng.integers(0, 8, 400)]).astype(dtype)
+    got = run(compile_spn(native, spn, dtype, **{"hip-kernel": kernel}), X)
+    check_f32(got, oracle_model(spn, dtype), X, False)
+    assert np.isneginf(got).any() and np.isfinite(got).any()
+
+
+def test_nan_handling(native):
+    from spnc import synthetic as syn
+    spn = syn.c2_spn()
+    X = syn.c2_inputs(64)
+    X[0, :] = np.nan          # everything marginalised: log 1
+    X[1, :8] = np.nan
+    for kernel in ("jit", "interpreter"):
+        got = run(compile_spn(native, spn, "float32", marginal=True, **{"hip-kernel": kernel}), X)
+        assert abs(got[0]) < 1e-6     # log of the weights summing to 1, in float32
+        check_f32(got, oracle_model(spn, "float32"), X, True)
+    # table leaves: NaN marginalises, a fractional value truncates, negative / too large is impossible
+    from spnc.structure import Categorical, Product
+    spn = Product(children=[Categorical(p=[0.25, 0.75], scope=0), Categorical(p=[0.1, 0.9], scope=1)])
+    X = np.array([[np.nan, 1.0], [1.9, np.nan], [np.nan, np.nan], [-0.5, 0.0], [-1.0, 0.0], [2.0, 0.0]])
+    want = [math.log(0.9), math.log(0.75), 0.0, math.log(0.25 * 0.1), -math.inf, -math.inf]
+    for kernel in ("jit", "interpreter"):
+        got = run(compile_spn(native, spn, "float64", marginal=True, **{"hip-kernel": kernel}), X)
+        assert np.allclose(got, want, rtol=0, atol=1e-6)
+
+
+def test_impossible_evidence_gives_minus_infinity(native):
+    """Zero-probability evidence under every child of a sum: -inf. (The reference's pairwise log-add
+    yields NaN for -inf + -inf, mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:233-239; the n-ary form does not.)"""
+    from spnc.structure import Categorical, Product, Sum
+    spn = Sum(weights=[0.5, 0.25, 0.25], children=[Product(children=[Categorical(p=[1.0, 0.0], scope=0), Categorical(p=[q, 1 - q], scope=1)])
+                                                   for q in (0.5, 0.25, 0.125)])
+    X = np.array([[1, 0], [0, 1]], dtype=np.int32)
+    for kernel in ("jit", "interpreter"):
+        got = run(compile_spn(native, spn, "int32", **{"hip-kernel": kernel}), X)
+        assert np.isneginf(got[0]) and abs(got[1] - math.log(0.5 * 0.5 + 0.25 * 0.75 + 0.25 * 0.875)) < 1e-6
+
+
+@pytest.mark.parametrize("n", [1, 63, 64, 255, 256, 257, 1023, 1025, 4097])
+def test_ragged_sizes(native, n):
+    from spnc import synthetic as syn
+    for cfg, opts in (("c1", {}), ("c2", {}), ("c2", {"hip-kernel": "interpreter"})):
+        c = syn.CONFIGS[cfg]
+        spn = c["spn"]()
+        X = c["inputs"](4097)[:n]
+        got = run(compile_spn(native, spn, c["dtype"], **opts), X)
+        full = ev.ll_reforder(oracle_model(spn, c["dtype"]), X, np.float32, marginal=False)
+        assert got.shape == (n,) and np.abs(got - full).max() <= F32_TOL
+
+
+def test_empty_batch_and_reuse(native):
+    from spnc import synthetic as syn
+    k = compile_spn(native, syn.c1_spn(), "int32")
+    assert k.execute(0, np.zeros((0, 6), dtype=np.int32)).shape == (0,)
+    X = syn.c1_inputs(100)
+    a, b = k.execute(100, X), k.execute(50, X[:50])      # compile once, execute many
+    assert np.array_equal(a[:50], b)
+    os.remove(k.fileName())
+
+
+def test_kernel_reloaded_from_file_computes_the_same(native):
+    from spnc import synthetic as syn
+    for cfg, opts in (("c3", {}), ("c3", {"hip-kernel": "interpreter"})):
+        c = syn.CONFIGS[cfg]
+        k = compile_spn(native, c["spn"](), c["dtype"], **opts)
+        X = c["inputs"](1000)
+        first = k.execute(1000, X)
+        again = native.Kernel(k.fileName()).execute(1000, X)
+        assert np.array_equal(first, again)
+        os.remove(k.fileName())
+
+
+def test_host_path_streams_large_batches_in_chunks(native):
+    """More rows than one staging chunk (32 MiB of input): chunk boundaries must not show."""
+    from spnc import synthetic as syn
+    spn = syn.c2_spn()
+    n = 1_300_000
+    X = np.tile(syn.c2_inputs(4096), (n // 4096 + 1, 1))[:n]
+    for opts in ({}, {"hip-kernel": "interpreter"}):
+        k = compile_spn(native, spn, "float32", **opts)
+        got = k.execute(n, X)
+        small = k.execute(4096, X[:4096])
+        os.remove(k.fileName())
+        assert np.abs(small - ev.ll_reforder(oracle_model(spn, "float32"), X[:4096], np.float32, marginal=False)).max() <= F32_TOL
+        reps = got[: (n // 4096) * 4096].reshape(-1, 4096)
+        assert np.array_equal(reps, np.broadcast_to(small, reps.shape))
+        assert np.array_equal(got[(n // 4096) * 4096:], small[: n % 4096])
+
+
+def test_device_pointer_checks(native):
+    import torch
+    from spnc import synthetic as syn
+    k = compile_spn(native, syn.c2_spn(), "float32")
+    x = torch.zeros(1024 * 16 + 4, dtype=torch.float32, device="cuda")
+    out = torch.empty(1024, dtype=torch.float32, device="cuda")
+    with pytest.raises(RuntimeError, match="input pointer must be aligned to 16 bytes"):
+        k.execute_device(1024, x.data_ptr() + 4, out.data_ptr())
+    k.execute_device(1024, x.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    os.remove(k.fileName())
+
+
+# ---- full benchmark sizes: properties that do not need the oracle at that size ----
+
+def test_c1_at_64m_rows_matches_the_729_state_table(native):
+    import torch
+    from spnc import synthetic as syn
+    k = compile_spn(native, syn.c1_spn(), "int32")
+    states = np.array(np.meshgrid(*[range(3)] * 6, indexing="ij")).reshape(6, -1).T.astype(np.int32)   # all 3^6 inputs
+    table = ev.ll_closed_f64(oracle_model(syn.c1_spn(), "int32"), states, marginal=False)
+    n = 64 * 2 ** 20
+    idx = torch.arange(n, device="cuda") % 729
+    x = torch.from_numpy(states).cuda()[idx].contiguous()
+    out = torch.empty(n, dtype=torch.float32, device="cuda")
+    k.execute_device(n, x.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    first = out[:729].cpu().numpy()
+    assert np.abs(first - table).max() <= F32_TOL
+    assert abs(np.exp(first.astype(np.float64)).sum() - 1.0) < 1e-5        # the distribution is normalised
+    assert bool((out == out[:729][idx]).all())                              # every row, bit for bit
+    os.remove(k.fileName())
+
+
+@pytest.mark.parametrize("cfg,opts", [("c2", {}), ("c5", {}), ("c3", {}), ("c4", {})])
+def test_full_size_batches_repeat_a_checked_block(native, cfg, opts):
+    import torch
+    from spnc import synthetic as syn
+    c = syn.CONFIGS[cfg]
+    spn = c["spn"]()
+    block = 3001 if cfg != "c4" else 1001          # odd, so repeats straddle tile and wave boundaries
+    Xb = c["inputs"](block)
+    n = c["n"]
+    k = compile_spn(native, spn, c["dtype"], marginal=c["marginal"], **opts)
+    want = ev.ll_reforder(oracle_model(spn, c["dtype"]), Xb, np.float32, marginal=c["marginal"])
+    idx = torch.arange(n, device="cuda") % block
+    x = torch.from_numpy(Xb).cuda()[idx].contiguous()
+    out = torch.empty(n, dtype=torch.float32, device="cuda")
+    k.execute_device(n, x.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert np.abs(out[:block].cpu().numpy() - want).max() <= F32_TOL
+    assert bool((out == out[:block][idx]).all())
+    os.remove(k.fileName())

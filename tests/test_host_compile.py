@@ -1,0 +1,203 @@
+"""Host layer through the C-ABI without a GPU: reader, validation, options, code generation, kernel files."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import rawfile as rf
+from conftest import GOLDEN, ROOT, compile_query, compile_spn, model_as_query, oracle_model, quiet
+
+QUERIES = ["categorical-example", "gaussian-example", "mini-example", "categorical6", "gaussian10", "histogram4", "NIPS5", "NIPS10",
+           "speaker_FADG0"]
+MODELS = ["nltcs", "plants", "fashion_mnist"]
+
+
+def test_library_exports_every_declared_symbol(native):
+    header = open(os.path.join(ROOT, "include", "spnc_hip.h")).read()
+    declared = re.findall(r"SPNC_HIP_API[^;(]*?\b(spnc_hip_\w+)\s*\(", header)
+    assert len(declared) == 9
+    lib = ctypes.CDLL(native.library_path())
+    for name in declared:
+        assert hasattr(lib, name), name
+
+
+def test_info_struct_layout_matches_header(native, tmp_path):
+    src = tmp_path / "sz.c"
+    src.write_text('#include <stdio.h>\n#include "spnc_hip.h"\nint main(){printf("%zu %zu", sizeof(spnc_hip_info), '
+                   '__builtin_offsetof(spnc_hip_info, flops_min));return 0;}\n')
+    exe = tmp_path / "sz"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), "-o", str(exe), str(src)], check=True)
+    size, off = map(int, subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split())
+    assert size == ctypes.sizeof(native._Info)
+    assert off == native._Info.flops_min.offset
+
+
+@pytest.mark.parametrize("name", QUERIES)
+def test_reference_query_files_compile(native, name):
+    from oracle import spn_model as sm
+    k = compile_query(native, os.path.join(GOLDEN, name + ".bin"))
+    q = sm.load(os.path.join(GOLDEN, name + ".bin"))
+    info = k.info()
+    assert os.path.isfile(k.fileName())
+    assert k.kernelName() == (q.model.name or "spn_kernel")
+    assert k.numFeatures() == q.model.num_features and k.batchSize() == q.batch_size
+    assert k.bytesPerFeature() == np.dtype(q.model.feature_type).itemsize
+    assert (k.numResults(), k.bytesPerResult(), k.dataType(), k.target(), k.queryType()) == (1, 4, "float32", 3, 1)
+    assert info["num_nodes"] <= len(q.model.nodes)
+    os.remove(k.fileName())
+
+
+@pytest.mark.parametrize("name", MODELS)
+def test_raw_models_are_rejected_then_compile_as_queries(native, name, tmp_path):
+    with pytest.raises(RuntimeError, match="Cannot compile raw models"):
+        compile_query(native, os.path.join(GOLDEN, name + ".bin"))
+    q = model_as_query(os.path.join(GOLDEN, name + ".bin"), "float64", str(tmp_path / "q.bin"))
+    k = compile_query(native, q)
+    info = k.info()
+    assert info["kernel_kind"] == (2 if name == "fashion_mnist" else 1)  # the 47k-node model goes to the interpreter
+    assert k.numFeatures() == {"nltcs": 16, "plants": 69, "fashion_mnist": 784}[name]
+    os.remove(k.fileName())
+
+
+def test_dedup_of_identical_leaves(native):
+    from spnc.structure import Gaussian, Product, Sum
+    a = Product(children=[Gaussian(0.0, 1.0, scope=0), Gaussian(1.0, 2.0, scope=1)])
+    b = Product(children=[Gaussian(0.0, 1.0, scope=0), Gaussian(2.0, 2.0, scope=1)])  # same first leaf, other object
+    k = compile_spn(native, Sum(weights=[0.5, 0.5], children=[a, b]), "float32")
+    assert k.info()["num_nodes"] == 6 and k.info()["num_gaussian"] == 3
+    os.remove(k.fileName())
+
+
+def test_algorithmic_counts(native):
+    from spnc import synthetic as syn
+    k = compile_spn(native, syn.c1_spn(), "int32")
+    i = k.info()
+    assert (i["flops_min"], i["trans_min"], i["num_categorical"], i["product_adds"]) == (5, 0, 6, 5)
+    os.remove(k.fileName())
+    k = compile_spn(native, syn.c2_spn(), "float32")
+    i = k.info()
+    # 1024 Gaussians * 4 + products (36 * 1 + 256 * 3) + 73 sums * 5k (k = 4); transcendentals 73 * (k + 1)
+    assert (i["num_gaussian"], i["num_product"], i["num_sum"]) == (1024, 292, 73)
+    assert (i["flops_min"], i["trans_min"]) == (4096 + 804 + 73 * 20, 73 * 5)
+    assert (i["flops_pairwise"], i["trans_pairwise"]) == (4096 + 804 + 73 * 25, 73 * 6)
+    os.remove(k.fileName())
+
+
+def test_option_handling(native):
+    path = os.path.join(GOLDEN, "NIPS5.bin")
+    with pytest.raises(RuntimeError, match="Unknown compile option bogus"):
+        compile_query(native, path, bogus=1)
+    with quiet(), pytest.raises(RuntimeError, match="Could not verify configuration constraints"):
+        native.SPNCompiler().compileQuery(path, {"use-log-space": "true"})  # target is required
+    with quiet(), pytest.raises(RuntimeError, match="only supports target 'HIP'"):
+        native.SPNCompiler().compileQuery(path, {"target": "CUDA"})
+    # options of the reference's CPU pipeline are accepted and ignored
+    k = compile_query(native, path, **{"cpu-vectorize": "true", "vector-library": "LIBMVEC", "use-shuffle": "true", "optLevel": 2})
+    os.remove(k.fileName())
+    with pytest.raises(RuntimeError, match="Could not parse option value"):
+        compile_query(native, path, **{"hip-kernel": "magic"})
+
+
+def test_graph_stats_file(native, tmp_path):
+    import json
+    out = tmp_path / "stats.json"
+    k = compile_query(native, os.path.join(GOLDEN, "NIPS5.bin"), **{"collect-graph-stats": "true", "graph-stats-file": str(out)})
+    st = json.load(open(out))
+    assert (st["featureCount"], st["sumCount"], st["productCount"], st["histogramCount"], st["innerCount"], st["leafCount"]) == (5, 1, 2, 10, 3, 10)
+    os.remove(k.fileName())
+
+
+def _bad(native, tmp_path, match, **kw):
+    path = rf.write(str(tmp_path / "bad.bin"), **kw)
+    with pytest.raises(RuntimeError, match=match):
+        compile_query(native, path)
+
+
+def test_validation_errors(native, tmp_path):
+    two = [rf.cat(1, 0), rf.cat(2, 1)]
+    _bad(native, tmp_path, "Can only deserialize joint queries", nodes=[], scope=[0], with_joint=False)
+    _bad(native, tmp_path, "No model attached to query", nodes=[], scope=[0], with_model=False)
+    _bad(native, tmp_path, "Cannot compile raw models", nodes=two + [rf.prod(0, [1, 2])], scope=[0, 1], header_kind=0)
+    _bad(native, tmp_path, "Leaf node references unknown feature", nodes=[rf.cat(1, 0), rf.cat(2, 7), rf.prod(0, [1, 2])], scope=[0, 1])
+    _bad(native, tmp_path, "No definition found for node with ID: 9", nodes=two + [rf.prod(0, [1, 9])], scope=[0, 1])
+    _bad(native, tmp_path, "No definition found for node with ID: 2", nodes=[rf.cat(1, 0), rf.prod(0, [1, 2]), rf.cat(2, 1)], scope=[0, 1])
+    _bad(native, tmp_path, "No definition found for node with ID: 5", nodes=two + [rf.prod(0, [1, 2])], scope=[0, 1], root=5)
+    _bad(native, tmp_path, "Unsupported feature data type complex64", nodes=two + [rf.prod(0, [1, 2])], scope=[0, 1], feature_type="complex64")
+    _bad(native, tmp_path, "Unsupported floating-point type float128", nodes=two + [rf.prod(0, [1, 2])], scope=[0, 1], feature_type="float128")
+    _bad(native, tmp_path, "Feature data type must be floating-point to support marginal", nodes=two + [rf.prod(0, [1, 2])],
+         scope=[0, 1], feature_type="int32", marginal=True)
+    _bad(native, tmp_path, "Weights must sum up to 1.0", nodes=[rf.cat(1, 0), rf.cat(2, 0), rf.wsum(0, [1, 2], [0.3, 0.8])], scope=[0])
+    _bad(native, tmp_path, "Number of weights must match", nodes=[rf.cat(1, 0), rf.cat(2, 0), rf.wsum(0, [1, 2], [1.0])], scope=[0])
+    _bad(native, tmp_path, "Number of addends must be greater than zero", nodes=[rf.wsum(0, [], [])], scope=[0])
+    _bad(native, tmp_path, "Number of operands must be at least one", nodes=[rf.prod(0, [])], scope=[0])
+    _bad(native, tmp_path, "Category probabilities should sum to 1.0", nodes=[rf.cat(0, 0, p=(0.5, 0.6))], scope=[0])
+    _bad(native, tmp_path, "Lower bound must be less or equal", nodes=[rf.hist(0, 0, breaks=(0, 3, 1), densities=(0.5, 0.5))], scope=[0])
+    _bad(native, tmp_path, "negative lower bound", nodes=[rf.hist(0, 0, breaks=(-1, 1, 2), densities=(0.5, 0.5))], scope=[0])
+    _bad(native, tmp_path, "does not match the size of the scope", nodes=[rf.cat(0, 0)], scope=[0], num_features=3)
+    with pytest.raises(RuntimeError, match="cannot open query file"):
+        compile_query(native, str(tmp_path / "missing.bin"))
+    (tmp_path / "junk.bin").write_bytes(b"\x00\x00\x00\x00\xff\xff\xff\x7f" + b"\x01" * 40)
+    with pytest.raises(RuntimeError, match="malformed Cap'n Proto"):
+        compile_query(native, str(tmp_path / "junk.bin"))
+
+
+def test_old_files_without_marginal_field(native, tmp_path):
+    """The reference's shipped query files encode JointProbability with an empty data section."""
+    path = rf.write(str(tmp_path / "old.bin"), nodes=[rf.cat(0, 0)], scope=[0], feature_type="int32", joint_data_words=0)
+    k = compile_query(native, path)  # would fail with 'floating-point to support marginal' if the default were true
+    os.remove(k.fileName())
+
+
+def test_scope_values_map_to_columns_in_ascending_order(native, tmp_path):
+    # scope values {5, 2}: column 0 is scope 2, column 1 is scope 5
+    path = rf.write(str(tmp_path / "s.bin"), nodes=[rf.cat(1, 5, p=(0.9, 0.1)), rf.cat(2, 2, p=(0.2, 0.8)), rf.prod(0, [1, 2])],
+                    scope=[5, 2], feature_type="int32")
+    k = compile_query(native, path)
+    src = k.source()
+    first = src.index("tab[0u + t1]")   # first table (scope 5) is indexed by column 1
+    second = src.index("u + t0]")       # second table (scope 2) by column 0
+    assert first < second
+    os.remove(k.fileName())
+
+
+def test_generated_source_variants(native):
+    from spnc import synthetic as syn
+    k = compile_spn(native, syn.c2_spn(), "float32")
+    src = k.source()
+    assert "__builtin_amdgcn_exp2f" in src and "spn_logadd" not in src and src.count("__builtin_amdgcn_logf") == 73
+    os.remove(k.fileName())
+    k = compile_spn(native, syn.c2_spn(), "float32", **{"hip-sum-form": "pairwise", "hip-log2-domain": "false"})
+    src = k.source()
+    assert src.count("spn_logadd(") == 73 * 3 + 1 and "log1pf(expf(b - a))" in src
+    os.remove(k.fileName())
+    k = compile_spn(native, syn.c2_spn(), "float32", marginal=True, **{"hip-compute-type": "float64"})
+    assert k.dataType() == "float64" and k.bytesPerResult() == 8 and "typedef double real_t;" in k.source()
+    os.remove(k.fileName())
+    k = compile_spn(native, syn.c2_spn(), "float64", **{"use-log-space": "false"})
+    assert k.dataType() == "float64" and "return log(" in k.source()
+    os.remove(k.fileName())
+    k = compile_spn(native, syn.c2_spn(), "float32", **{"hip-kernel": "interpreter"})
+    assert k.info()["kernel_kind"] == 2 and "sumlayer" not in k.source() and "sum(4 terms)" in k.source()
+    os.remove(k.fileName())
+    k = compile_spn(native, syn.c4_spn(), "float32")
+    assert k.info()["kernel_kind"] == 2 and "sumlayer(8 sums x 64 terms)" in k.source()
+    os.remove(k.fileName())
+
+
+def test_kernel_file_round_trip(native):
+    from spnc import synthetic as syn
+    for opts in ({}, {"hip-kernel": "interpreter"}):
+        k = compile_spn(native, syn.c3_spn(), "int32", **opts)
+        k2 = native.Kernel(k.fileName(), k.kernelName(), k.queryType(), k.target(), k.batchSize(), k.numFeatures(), k.bytesPerFeature(),
+                           k.numResults(), k.bytesPerResult(), k.dataType())
+        assert k2.info() == k.info() and k2.source() == k.source()
+        with pytest.raises(RuntimeError, match="holds numFeatures"):
+            native.Kernel(k.fileName(), k.kernelName(), 1, 3, k.batchSize(), 7, 4, 1, 4, "float32")
+        os.remove(k.fileName())
+    with pytest.raises(RuntimeError, match="cannot open kernel file"):
+        native.Kernel("/nonexistent/kernel.hipk")
+    with pytest.raises(RuntimeError, match="not a spnc-hip kernel file"):
+        native.Kernel(os.path.join(GOLDEN, "NIPS5.bin"))
