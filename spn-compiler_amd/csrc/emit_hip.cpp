@@ -65,9 +65,15 @@ struct Emitter {
     // (mlir/lib/Conversion/HiSPNtoLoSPN/NodePatterns.cpp:17-40,49-88).
     size_t k = hi - lo;
     if (k == 1) return leaf(lo);
-    if (k == 2) return comb(leaf(lo), leaf(lo + 1));
+    if (k == 2) {
+      auto a = leaf(lo);  // sequenced: the callbacks emit code
+      auto b = leaf(lo + 1);
+      return comb(a, b);
+    }
     size_t pivot = lo + (k + 1) / 2;
-    return comb(tree(lo, pivot, leaf, comb), tree(pivot, hi, leaf, comb));
+    auto l = tree(lo, pivot, leaf, comb);
+    auto r = tree(pivot, hi, leaf, comb);
+    return comb(l, r);
   }
 
   void prepare() {
