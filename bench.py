@@ -81,20 +81,31 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None):
     slots = flops + 3 * trans
     props = torch.cuda.get_device_properties(device)
     clock_hz = props.clock_rate * 1e3 if hasattr(props, "clock_rate") else 2.4e9
-    valu_peak = props.multi_processor_count * 64 * clock_hz  # lane-operations per second
+    # FP32 VALU issue rate: 128 lane-operations per CU per clock (a wave64 instruction issues in
+    # two cycles on each of the four SIMDs). This is what the published 157.3 TFLOP/s is made of
+    # (256 CUs x 128 lanes x 2 flops per FMA x 2.4 GHz); a transcendental takes four such slots.
+    valu_peak = props.multi_processor_count * 128 * clock_hz  # lane-operations per second
     t_launch = launch_ms * 1e-3
     hbm_gbs = bytes_per_sample * n / t_launch / 1e9
     tflops = flops * n / t_launch / 1e12
     t_min_hbm = bytes_per_sample * n / (HBM_PEAK_GBS * 1e9)
     t_min_valu = slots * n / valu_peak
     hbm_bound = t_min_hbm >= t_min_valu
+    # Compute-bound kernels are priced in issue slots (simple op 1, transcendental 4) against the
+    # FP32 vector peak for single-flop instructions, i.e. half the published FMA figure.
+    slot_tflops = slots * n / t_launch / 1e12
+    slot_peak = FP32_VECTOR_PEAK_TFLOPS / 2
     roof = {
         "bound": "hbm" if hbm_bound else "valu-fp32",
-        "achieved": round(hbm_gbs if hbm_bound else tflops, 3),
-        "peak": HBM_PEAK_GBS if hbm_bound else FP32_VECTOR_PEAK_TFLOPS,
+        "achieved": round(hbm_gbs if hbm_bound else slot_tflops, 3),
+        "peak": HBM_PEAK_GBS if hbm_bound else slot_peak,
         "unit": "GB/s" if hbm_bound else "TFLOP/s",
-        "frac": round((hbm_gbs / HBM_PEAK_GBS) if hbm_bound else (tflops / FP32_VECTOR_PEAK_TFLOPS), 4),
+        "frac": round((hbm_gbs / HBM_PEAK_GBS) if hbm_bound else (slot_tflops / slot_peak), 4),
         "traffic": None,
+        "peak_note": ("published HBM3E bandwidth" if hbm_bound else
+                      "published FP32 vector peak 157.3 TFLOP/s counts an FMA as 2 flops; this path issues single-flop "
+                      "instructions, so the ceiling is 78.65 T issue slots/s; achieved = (flops + 3*transcendentals) per sample"),
+        "fma_flops_tflops": round(tflops, 3),
         "kernel": "spn_kernel (hipRTC straight-line)" if info["kernel_kind"] == 1 else "spn_interp_kernel",
         "launch_ms": round(launch_ms, 4),
         "bytes_per_sample": bytes_per_sample,
@@ -162,6 +173,9 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="measure only the selected configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--opt", action="append", default=[], help="extra compiler option key=value")
+    ap.add_argument("--copy-gib", type=float, default=0.0,
+                    help="instead of the benchmark, run a plain device-to-device copy of this many GiB per step "
+                         "(reference point for rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: samples are independent, a multi-GPU run would only split the batch; use --gpus 1",
@@ -174,6 +188,21 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     device = torch.device("cuda:0")
+    if args.copy_gib > 0:
+        nbytes = int(args.copy_gib * 2 ** 30)
+        a = torch.ones(nbytes // 4, dtype=torch.float32, device=device)
+        b = torch.empty_like(a)
+        for _ in range(args.warmup):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+        print(json.dumps({"mode": "copy", "bytes_read_per_step": nbytes, "bytes_written_per_step": nbytes, "steps": args.steps,
+                          "ms_per_step": dt * 1e3, "GB/s": 2 * nbytes / dt / 1e9}))
+        return
     extra = dict(kv.split("=", 1) for kv in args.opt)
     log = io.StringIO()
     with contextlib.redirect_stdout(log):

@@ -5,6 +5,7 @@
 #include <cstdio>
 #include <sstream>
 #include <stdexcept>
+#include <unordered_map>
 #include <vector>
 
 namespace spnc_hip {
@@ -26,6 +27,7 @@ struct Emitter {
   std::vector<bool> featUsed;
   std::vector<bool> featPrepared;
   std::vector<bool> emitted;
+  std::unordered_map<uint32_t, double> foldedWeight;
   bool vectorRows = true;
 
   Emitter(const Graph& graph, const CompileOptions& opts) : g(graph), o(opts) {
@@ -156,6 +158,62 @@ struct Emitter {
     }
   }
 
+  // A Gaussian leaf read by exactly one product is evaluated inside that product.
+  bool inlineLeaf(uint32_t c) const { return g.nodes[c].kind == NodeKind::Gaussian && g.nodes[c].uses == 1; }
+  bool fusableProduct(uint32_t i) const {
+    if (g.nodes[i].kind != NodeKind::Product) return false;
+    for (uint32_t c : g.nodes[i].children)
+      if (inlineLeaf(c)) return true;
+    return false;
+  }
+
+  // Log-space product with Gaussian leaves folded in. A leaf's value coef + d*d*den (d = x - mean)
+  // is rewritten den * (d*d + coef/den), so that leaf plus accumulation cost three instructions
+  // whose constants are all literals: d = x - mean; t = fma(d, d, coef/den); acc = fma(t, den, acc).
+  // A log-weight handed down by the single parent sum is folded into the first leaf's constant.
+  // With marginal support a NaN input selects the constant that makes the leaf contribute 0.
+  void emitFusedProduct(uint32_t i) {
+    const auto& n = g.nodes[i];
+    std::vector<uint32_t> leaves, rest;
+    for (uint32_t c : n.children) (inlineLeaf(c) ? leaves : rest).push_back(c);
+    double fold = 0.0;
+    auto it = foldedWeight.find(i);
+    if (it != foldedWeight.end()) fold = it->second;
+    std::string p = "p" + std::to_string(i) + "_";
+    std::string acc;
+    if (!rest.empty()) {
+      std::string e = tree(
+          0, rest.size(),
+          [&](size_t k) {
+            emitNode(rest[k]);
+            return v(rest[k]);
+          },
+          [&](const std::string& a, const std::string& b) { return "(" + a + " + " + b + ")"; });
+      acc = p + "r";
+      body << "  const real_t " << acc << " = " << e << ";\n";
+    }
+    const char* fma = f64 ? "__builtin_fma(" : "__builtin_fmaf(";
+    for (size_t k = 0; k < leaves.size(); ++k) {
+      const auto& leaf = g.nodes[leaves[k]];
+      emitFeaturePrep(leaf.feature);
+      const std::string x = "g" + std::to_string(leaf.feature);
+      const double den = -(1.0 / (2.0 * leaf.stddev * leaf.stddev)) * scale;
+      const double coef = (-std::log(leaf.stddev) + -0.5 * std::log(2 * M_PI)) * scale;
+      const double extra = k == 0 ? fold / den : 0.0;
+      const std::string d = p + "d" + std::to_string(k), t = p + "t" + std::to_string(k), a = p + "a" + std::to_string(k);
+      body << "  const real_t " << d << " = " << x << " - " << lit(leaf.mean) << ";\n";
+      if (g.supportMarginal)
+        body << "  const real_t " << t << " = (" << x << " != " << x << ") ? " << lit(extra) << " : " << fma << d << ", " << d << ", "
+             << lit(coef / den + extra) << ");\n";
+      else
+        body << "  const real_t " << t << " = " << fma << d << ", " << d << ", " << lit(coef / den + extra) << ");\n";
+      if (acc.empty()) body << "  const real_t " << a << " = " << t << " * " << lit(den) << ";\n";
+      else body << "  const real_t " << a << " = " << fma << t << ", " << lit(den) << ", " << acc << ");\n";
+      acc = a;
+    }
+    body << "  const real_t " << v(i) << " = " << acc << ";\n";
+  }
+
   // Emits node i after everything it depends on. Children are emitted lazily, right before
   // their first use, so that a sum over hundreds of children never holds all of them live.
   void emitNode(uint32_t i) {
@@ -185,6 +243,10 @@ struct Emitter {
         body << "  const real_t " << v(i) << " = tab[" << tableOffset[i] << "u + t" << n.feature << "];\n";
         break;
       case NodeKind::Product: {
+        if (logSpace && fusableProduct(i)) {
+          emitFusedProduct(i);
+          break;
+        }
         const char* op = logSpace ? " + " : " * ";
         std::string e = tree(
             0, n.children.size(),
@@ -226,8 +288,15 @@ struct Emitter {
       return;
     }
     auto term = [&](size_t j) {
-      emitNode(n.children[j]);
-      return fresh(v(n.children[j]) + " + " + lit(logConst(n.weights[j])));
+      const uint32_t c = n.children[j];
+      const double w = logConst(n.weights[j]);
+      if (!emitted[c] && g.nodes[c].uses == 1 && fusableProduct(c) && std::isfinite(w)) {
+        foldedWeight[c] = w;  // the child adds the log-weight itself
+        emitNode(c);
+        return v(c);
+      }
+      emitNode(c);
+      return fresh(v(c) + " + " + lit(w));
     };
     if (k == 1) {
       body << "  const real_t " << v(i) << " = " << term(0) << ";\n";
@@ -302,11 +371,11 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   const unsigned vw = vb / eb;
   js.inputAlign = vb;
 
+  // Samples per lane: two independent samples give the scheduler more to overlap; kernels that
+  // are heavy on registers (large LDS tables, NaN selects) stay at one.
+  const size_t work = g.nodes.size() + g.stats.sumTerms;
   unsigned U = unsigned(o.samplesPerLane);
-  if (U == 0) {
-    size_t work = g.nodes.size() + g.stats.sumTerms;
-    U = work <= 48 ? 4 : (work <= 400 ? 2 : 1);
-  }
+  if (U == 0) U = (work <= 4000 && !g.supportMarginal && size_t(js.tableEntries) * realBytes <= 16 * 1024) ? 2 : 1;
   if (!e.vectorRows) U = 1;
   js.samplesPerLane = U;
 
@@ -322,12 +391,15 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     for (size_t i = 0; i < e.tablePool.size(); ++i) s << (i ? ", " : "") << (i % 8 == 0 ? "\n  " : "") << e.lit(e.tablePool[i]);
     s << "};\n";
   }
+  // Out-of-line library math keeps hipRTC times in seconds for large graphs; small graphs inline it.
+  const bool inlineMath = g.nodes.size() + g.stats.sumTerms <= 4000;
+  const char* mathAttr = inlineMath ? "__forceinline__" : "__attribute__((noinline))";
   if (!e.log2Dom) {
-    s << "static __device__ __attribute__((noinline)) real_t spn_exp(real_t x) { return " << (e.f64 ? "exp(x)" : "expf(x)") << "; }\n";
-    s << "static __device__ __attribute__((noinline)) real_t spn_log(real_t x) { return " << (e.f64 ? "log(x)" : "logf(x)") << "; }\n";
+    s << "static __device__ " << mathAttr << " real_t spn_exp(real_t x) { return " << (e.f64 ? "exp(x)" : "expf(x)") << "; }\n";
+    s << "static __device__ " << mathAttr << " real_t spn_log(real_t x) { return " << (e.f64 ? "log(x)" : "logf(x)") << "; }\n";
   }
   if (e.logSpace && o.sumForm == SumForm::Pairwise) {
-    s << "static __device__ " << (e.log2Dom ? "__forceinline__" : "__attribute__((noinline))") << " real_t spn_logadd(real_t x, real_t y) {\n"
+    s << "static __device__ " << (e.log2Dom ? "__forceinline__" : mathAttr) << " real_t spn_logadd(real_t x, real_t y) {\n"
          "  const bool gt = x > y;\n  const real_t a = gt ? x : y;\n  const real_t b = gt ? y : x;\n";
     if (e.f64) s << "  return a + log1p(exp(b - a));\n";
     else if (e.log2Dom) s << "  return a + __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(b - a));\n";
@@ -378,9 +450,55 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   } else {
     s << "  const real_t* tab = nullptr;\n";
   }
-  s << "  const unsigned long long tile = (unsigned long long)SPN_BLOCK * SPN_U;\n"
-       "  for (unsigned long long base = blockIdx.x * tile; base < n; base += gridDim.x * tile) {\n";
-  if (U == 1) {
+  // "gpu-shared-mem": the block copies its tile of rows from HBM into LDS with fully coalesced
+  // 16-byte loads, then every lane reads its own rows from LDS. Same role as the reference's
+  // shared-memory preload (mlir/lib/Dialect/LoSPN/Passes/LoSPNGPUSharedMemoryInsertion.cpp:99-260)
+  // and, like there, skipped when the tile does not fit.
+  const size_t tileBytes = size_t(js.blockSize) * U * rowBytes;
+  const size_t ldsTables = js.tablesInLds ? size_t(js.tableEntries) * realBytes : 0;
+  // Without an explicit option the tile is staged when the kernel is closer to the HBM bound
+  // than to the VALU bound (about 6.4e12 B/s against 6e13 lane-operations/s on MI355X).
+  const double tHbm = double(rowBytes + realBytes) / 6.4e12, tValu = double(g.stats.issueSlotsMin()) / 6.0e13;
+  const bool wantStaged = o.gpuSharedMem < 0 ? tHbm > 0.5 * tValu : o.gpuSharedMem == 1;
+  const bool staged = wantStaged && e.vectorRows && tileBytes % 16 == 0 && tileBytes + ldsTables <= 64 * 1024;
+  js.stagedInput = staged;
+  // Blocks with next to no set-up take one tile each; blocks that stage tables stay resident.
+  js.oneTilePerBlock = js.tableEntries <= 256;
+  if (staged) js.inputAlign = 16;
+  s << "  const unsigned long long tile = (unsigned long long)SPN_BLOCK * SPN_U;\n";
+  if (staged)
+    s << "  typedef unsigned int spn_v4 __attribute__((ext_vector_type(4)));\n"
+         "  __shared__ __attribute__((aligned(16))) feat_t spn_tile[SPN_BLOCK * SPN_U * SPN_F];\n";
+  s << "  for (unsigned long long base = blockIdx.x * tile; base < n; base += gridDim.x * tile) {\n";
+  const char* tail =
+      "      for (int u = 0; u < SPN_U; ++u) {\n"
+      "        const unsigned long long i = base + (unsigned long long)u * SPN_BLOCK + threadIdx.x;\n"
+      "        if (i < n) {\n"
+      "          feat_t x[SPN_F];\n"
+      "          spn_load_row(in, i, x);\n"
+      "          out[i] = spn_eval(x, tab);\n"
+      "        }\n"
+      "      }\n";
+  if (staged) {
+    s << "    if (base + tile <= n) {\n"
+         "      const spn_v4* src = reinterpret_cast<const spn_v4*>(in + base * SPN_F);\n"
+         "      spn_v4* dst = reinterpret_cast<spn_v4*>(spn_tile);\n"
+         "      constexpr unsigned NV = SPN_BLOCK * SPN_U * SPN_F * sizeof(feat_t) / 16;\n"
+         "#pragma unroll\n"
+         "      for (unsigned v = threadIdx.x; v < NV; v += SPN_BLOCK) dst[v] = __builtin_nontemporal_load(src + v);\n"
+         "      __syncthreads();\n"
+         "      feat_t x[SPN_U][SPN_F];\n"
+         "#pragma unroll\n"
+         "      for (int u = 0; u < SPN_U; ++u)\n"
+         "#pragma unroll\n"
+         "        for (int f = 0; f < SPN_F; ++f) x[u][f] = spn_tile[(u * SPN_BLOCK + threadIdx.x) * SPN_F + f];\n"
+         "      __syncthreads();\n"
+         "#pragma unroll\n"
+         "      for (int u = 0; u < SPN_U; ++u)\n"
+         "        __builtin_nontemporal_store(spn_eval(x[u], tab), out + base + (unsigned long long)u * SPN_BLOCK + threadIdx.x);\n"
+         "    } else {\n"
+      << tail << "    }\n";
+  } else if (U == 1) {
     s << "    const unsigned long long i = base + threadIdx.x;\n"
          "    if (i < n) {\n";
     if (e.vectorRows)
@@ -399,15 +517,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
          "      for (int u = 0; u < SPN_U; ++u)\n"
          "        __builtin_nontemporal_store(spn_eval(x[u], tab), out + base + (unsigned long long)u * SPN_BLOCK + threadIdx.x);\n"
          "    } else {\n"
-         "      for (int u = 0; u < SPN_U; ++u) {\n"
-         "        const unsigned long long i = base + (unsigned long long)u * SPN_BLOCK + threadIdx.x;\n"
-         "        if (i < n) {\n"
-         "          feat_t x[SPN_F];\n"
-         "          spn_load_row(in, i, x);\n"
-         "          out[i] = spn_eval(x, tab);\n"
-         "        }\n"
-         "      }\n"
-         "    }\n";
+      << tail << "    }\n";
   }
   s << "  }\n"
        "}\n";

@@ -21,6 +21,8 @@ struct JitSource {
   unsigned bytesPerResult = 4;
   unsigned tableEntries = 0;  // entries of the leaf-table pool (0 = none)
   bool tablesInLds = false;
+  bool oneTilePerBlock = false;
+  bool stagedInput = false;   // rows reach the lanes through an LDS tile ("gpu-shared-mem")
 };
 
 JitSource emitHipSource(const Graph& g, const CompileOptions& o);

@@ -25,12 +25,15 @@ struct InterpLaunch {
 };
 
 // Enqueues the interpreter on `stream`. ldsBytes = ldsSlots * INTERP_BLOCK * sizeof(compute type).
-hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain, unsigned grid, size_t ldsBytes, hipStream_t stream);
+// mode 0: all slots in LDS; 1: the program's short pool in LDS, flagged instructions may touch the spill tier;
+// 2: any instruction may touch the spill tier.
+hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain, int mode, unsigned grid, size_t ldsBytes,
+                             hipStream_t stream);
 
 // Largest dynamic LDS size a block of the interpreter may request on the current device.
 hipError_t interpreterMaxLds(bool f64, bool log2Domain, size_t* bytes);
 
 // Resident blocks per CU for a given dynamic LDS size.
-hipError_t interpreterOccupancy(bool f64, bool log2Domain, size_t ldsBytes, int* blocksPerCU);
+hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, size_t ldsBytes, int* blocksPerCU);
 
 }  // namespace spnc_hip

@@ -41,7 +41,32 @@ struct Builder {
 
 }  // namespace
 
+namespace {
+InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t longRange);
+}
+
+// Values that stay live for more than `longRange` instructions are numbered after all the others
+// ("long pool"), so that the launcher can keep the busy, short-lived slots in LDS and the rarely
+// touched long-lived ones in the spill tier. The range is lowered until the short pool fits the
+// LDS share that lets two blocks reside on a CU.
 InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
+  const uint32_t target = o.computeType == ComputeType::F64 ? 36 : 72;
+  InterpProgram best;
+  bool have = false;
+  for (uint32_t range : {0xffffffffu, 512u, 256u, 128u, 64u, 32u, 16u, 8u}) {
+    InterpProgram p = buildWithRange(g, o, range);
+    const bool fits = p.shortSlots <= target;
+    if (!have || p.shortSlots < best.shortSlots) {
+      best = std::move(p);
+      have = true;
+    }
+    if (fits) break;
+  }
+  return best;
+}
+
+namespace {
+InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t longRange) {
   if (!o.useLogSpace) throw std::runtime_error("The interpreter kernel supports log-space computation only");
   InterpProgram p;
   p.f64 = o.computeType == ComputeType::F64;
@@ -101,6 +126,57 @@ InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
     if (isLeaf(i) && g.nodes[i].uses == 1 && soleParent[i] != NONE && g.nodes[soleParent[i]].kind == NodeKind::Product)
       inlined[i] = true;
 
+  // Sums over a complete outer product: the sums of a group share the child list
+  // [prod(a_0,b_0), prod(a_0,b_1), ..., prod(a_NA-1,b_NB-1)] and nobody else reads those products.
+  // Then exp(a_r + b_c - m) = exp(a_r - ma) * exp(b_c - mb) and the products need not exist.
+  struct Outer {
+    std::vector<uint32_t> a, b;
+  };
+  std::map<std::vector<uint32_t>, Outer> outerOf;
+  std::vector<bool> absorbed(N, false);
+  {
+    std::map<std::vector<uint32_t>, uint32_t> groupSize;
+    for (uint32_t i = 0; i < N; ++i)
+      if (g.nodes[i].kind == NodeKind::Sum && g.nodes[i].children.size() >= 4) groupSize[g.nodes[i].children]++;
+    for (const auto& entry : groupSize) {
+      const std::vector<uint32_t>& kids = entry.first;
+      const uint32_t members = entry.second;
+      bool ok = true;
+      for (uint32_t c : kids) {
+        const auto& pn = g.nodes[c];
+        if (pn.kind != NodeKind::Product || pn.children.size() != 2 || pn.uses != members || inlined[pn.children[0]] ||
+            inlined[pn.children[1]]) {
+          ok = false;
+          break;
+        }
+      }
+      if (!ok) continue;
+      size_t nb = 1;
+      while (nb < kids.size() && g.nodes[kids[nb]].children[0] == g.nodes[kids[0]].children[0]) ++nb;
+      if (kids.size() % nb != 0) continue;
+      const size_t na = kids.size() / nb;
+      if ((nb != 2 && nb != 4 && nb != 8 && nb != 16) || na < 2 || na > 64) continue;
+      Outer o;
+      for (size_t r = 0; r < na; ++r) o.a.push_back(g.nodes[kids[r * nb]].children[0]);
+      for (size_t c = 0; c < nb; ++c) o.b.push_back(g.nodes[kids[c]].children[1]);
+      for (size_t r = 0; r < na && ok; ++r)
+        for (size_t c = 0; c < nb; ++c) {
+          const auto& pn = g.nodes[kids[r * nb + c]];
+          if (pn.children[0] != o.a[r] || pn.children[1] != o.b[c]) {
+            ok = false;
+            break;
+          }
+        }
+      // A child list naming one product twice would make the use counts above meaningless.
+      std::vector<uint32_t> sorted = kids;
+      std::sort(sorted.begin(), sorted.end());
+      if (std::adjacent_find(sorted.begin(), sorted.end()) != sorted.end()) ok = false;
+      if (!ok) continue;
+      for (uint32_t c : kids) absorbed[c] = true;
+      outerOf[kids] = std::move(o);
+    }
+  }
+
   struct Instr {
     InterpOp op;
     std::vector<uint32_t> defs;  // graph nodes whose values this instruction writes
@@ -113,10 +189,28 @@ InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
     if (g.nodes[i].kind == NodeKind::Sum && g.nodes[i].children.size() >= 2) layerOf[g.nodes[i].children].push_back(i);
   std::vector<bool> emitted(N, false);
   for (uint32_t i = 0; i < N; ++i) {
-    if (emitted[i] || inlined[i]) continue;
+    if (emitted[i] || inlined[i] || absorbed[i]) continue;
     const auto& n = g.nodes[i];
     if (n.kind == NodeKind::Sum && n.children.size() >= 2) {
       const std::vector<uint32_t>& group = layerOf[n.children];
+      auto outer = outerOf.find(n.children);
+      if (outer != outerOf.end()) {
+        std::vector<uint32_t> srcs = outer->second.a;
+        srcs.insert(srcs.end(), outer->second.b.begin(), outer->second.b.end());
+        size_t pos = 0;
+        while (pos < group.size()) {
+          size_t left = group.size() - pos;
+          size_t m = left >= 8 ? 8 : (left >= 4 ? 4 : (left >= 2 ? 2 : 1));
+          Instr in{OP_OUTERSUM, {}, srcs, group[pos]};
+          for (size_t j = 0; j < m; ++j) {
+            in.defs.push_back(group[pos + j]);
+            emitted[group[pos + j]] = true;
+          }
+          instrs.push_back(std::move(in));
+          pos += m;
+        }
+        continue;
+      }
       // Split the group into layers of 8, 4, 2 sums and single sums.
       size_t pos = 0;
       while (pos < group.size()) {
@@ -148,17 +242,31 @@ InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
   for (uint32_t k = 0; k < instrs.size(); ++k)
     for (uint32_t s : instrs[k].srcs) lastUse[s] = k;
   lastUse[g.root()] = uint32_t(instrs.size());  // read by OP_END
+  std::vector<uint32_t> firstDef(N, 0);
+  for (uint32_t k = 0; k < instrs.size(); ++k)
+    for (uint32_t d : instrs[k].defs) firstDef[d] = k;
+  constexpr uint32_t LONG_BIT = 0x80000000u;  // marks long-pool slot numbers until they are renumbered
   std::vector<uint32_t> slotOf(N, NONE);
-  std::priority_queue<uint32_t, std::vector<uint32_t>, std::greater<uint32_t>> freeSlots;
-  uint32_t highWater = nextSlot;
-  auto allocSlot = [&]() {
-    if (!freeSlots.empty()) {
-      uint32_t s = freeSlots.top();
-      freeSlots.pop();
+  typedef std::priority_queue<uint32_t, std::vector<uint32_t>, std::greater<uint32_t>> MinHeap;
+  MinHeap freeShort, freeLong;
+  uint32_t highWater = nextSlot, longCount = 0;
+  auto allocSlot = [&](uint32_t node) {
+    const bool isLong = lastUse[node] - firstDef[node] > longRange;
+    MinHeap& heap = isLong ? freeLong : freeShort;
+    if (!heap.empty()) {
+      uint32_t s = heap.top();
+      heap.pop();
       return s;
     }
-    return highWater++;
+    return isLong ? (LONG_BIT | longCount++) : highWater++;
   };
+  auto releaseSlot = [&](uint32_t s) { ((s & LONG_BIT) ? freeLong : freeShort).push(s); };
+  std::vector<size_t> longWords;  // positions in p.code holding long-pool slot numbers
+  auto slotWord = [&](uint32_t s) {
+    if (s & LONG_BIT) longWords.push_back(p.code.size());
+    b.word(s);
+  };
+  auto slotName = [&](uint32_t s) { return (s & LONG_BIT) ? "L" + std::to_string(s & ~LONG_BIT) : "s" + std::to_string(s); };
 
   auto emitInlineLeaf = [&](uint32_t c) {
     const auto& leaf = g.nodes[c];
@@ -185,9 +293,13 @@ InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
       std::sort(uniq.begin(), uniq.end());
       uniq.erase(std::unique(uniq.begin(), uniq.end()), uniq.end());
       for (uint32_t s : uniq)
-        if (lastUse[s] == k) freeSlots.push(slotOf[s]);
+        if (lastUse[s] == k) releaseSlot(slotOf[s]);
     }
-    for (uint32_t d : in.defs) slotOf[d] = allocSlot();
+    for (uint32_t d : in.defs) slotOf[d] = allocSlot(d);
+    // Bit 7 of the opcode tells the kernel that this instruction touches the long pool.
+    uint32_t longFlag = 0;
+    for (uint32_t d : in.defs) longFlag |= (slotOf[d] & LONG_BIT) ? 0x80u : 0u;
+    for (uint32_t sidx : in.srcs) longFlag |= (slotOf[sidx] & LONG_BIT) ? 0x80u : 0u;
     const auto& n = g.nodes[in.node];
     switch (in.op) {
       case OP_PROD: {
@@ -198,40 +310,58 @@ InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
           for (uint32_t c : n.children)
             if (inlined[c]) (isTable(c) ? ts : gs).push_back(c);
         }
-        b.word(OP_PROD);
-        b.word(slotOf[in.node]);
+        b.word(OP_PROD | longFlag);
+        slotWord(slotOf[in.node]);
         b.word(uint32_t(in.srcs.size()));
         b.word(uint32_t(gs.size()));
         b.word(uint32_t(ts.size()));
-        for (uint32_t s : in.srcs) b.word(slotOf[s]);
+        for (uint32_t s : in.srcs) slotWord(slotOf[s]);
         for (uint32_t c : gs) emitInlineLeaf(c);
         for (uint32_t c : ts) emitInlineLeaf(c);
-        b.txt << "  s" << slotOf[in.node] << " = prod(" << in.srcs.size() << " slots, " << gs.size() << " gaussians, " << ts.size()
+        b.txt << "  " << slotName(slotOf[in.node]) << " = prod(" << in.srcs.size() << " slots, " << gs.size() << " gaussians, " << ts.size()
               << " tables)   ; node " << in.node << "\n";
         break;
       }
       case OP_SUM: {
         uint32_t cnt = uint32_t(n.children.size());
-        b.word(OP_SUM | (cnt << 8));
-        b.word(slotOf[in.node]);
+        b.word(OP_SUM | longFlag | (cnt << 8));
+        slotWord(slotOf[in.node]);
         for (uint32_t j = 0; j < cnt; ++j) {
-          b.word(slotOf[n.children[j]]);
+          slotWord(slotOf[n.children[j]]);
           if (cnt == 1) b.real(b.logConst(n.weights[j]));  // single child: value + log weight
           else b.real(n.weights[j]);
         }
-        b.txt << "  s" << slotOf[in.node] << " = sum(" << cnt << " terms)   ; node " << in.node << "\n";
+        b.txt << "  " << slotName(slotOf[in.node]) << " = sum(" << cnt << " terms)   ; node " << in.node << "\n";
         break;
       }
       case OP_SUMLAYER: {
         uint32_t cnt = uint32_t(n.children.size());
         uint32_t m = uint32_t(in.defs.size());
-        b.word(OP_SUMLAYER | (cnt << 8));
+        b.word(OP_SUMLAYER | longFlag | (cnt << 8));
         b.word(m);
-        for (uint32_t d : in.defs) b.word(slotOf[d]);
-        for (uint32_t j = 0; j < cnt; ++j) b.word(slotOf[n.children[j]]);
+        for (uint32_t d : in.defs) slotWord(slotOf[d]);
+        for (uint32_t j = 0; j < cnt; ++j) slotWord(slotOf[n.children[j]]);
         for (uint32_t j = 0; j < cnt; ++j)
           for (uint32_t d : in.defs) b.real(g.nodes[d].weights[j]);
-        b.txt << "  s" << slotOf[in.defs[0]] << ".. = sumlayer(" << m << " sums x " << cnt << " terms)   ; nodes " << in.defs[0] << "..\n";
+        b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = sumlayer(" << m << " sums x " << cnt << " terms)   ; nodes " << in.defs[0] << "..\n";
+        break;
+      }
+      case OP_OUTERSUM: {
+        const Outer& o = outerOf.at(n.children);
+        const uint32_t na = uint32_t(o.a.size()), nb = uint32_t(o.b.size());
+        uint32_t m = uint32_t(in.defs.size());
+        // A single leftover sum is encoded as a layer of two identical sums writing the same slot.
+        std::vector<uint32_t> defs = in.defs;
+        if (m == 1) defs.push_back(in.defs[0]);
+        b.word(OP_OUTERSUM | longFlag | (na << 8) | (nb << 16));
+        b.word(uint32_t(defs.size()));
+        for (uint32_t d : defs) slotWord(slotOf[d]);
+        for (uint32_t a : o.a) slotWord(slotOf[a]);
+        for (uint32_t c : o.b) slotWord(slotOf[c]);
+        for (uint32_t j = 0; j < na * nb; ++j)
+          for (uint32_t d : defs) b.real(g.nodes[d].weights[j]);
+        b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = outersum(" << m << " sums x " << na << "x" << nb << " products)   ; nodes " << in.defs[0]
+              << "..\n";
         break;
       }
       default:
@@ -239,18 +369,21 @@ InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
     }
     // A value nobody reads later (cannot happen for reachable nodes, kept for safety).
     for (uint32_t d : in.defs)
-      if (d != g.root() && lastUse[d] <= k) freeSlots.push(slotOf[d]);
+      if (d != g.root() && lastUse[d] <= k) releaseSlot(slotOf[d]);
   }
-  b.word(OP_END);
-  b.word(slotOf[g.root()]);
-  p.numSlots = highWater;
+  b.word(OP_END | ((slotOf[g.root()] & LONG_BIT) ? 0x80u : 0u));
+  slotWord(slotOf[g.root()]);
+  for (size_t pos : longWords) p.code[pos] = highWater + (p.code[pos] & ~LONG_BIT);
+  p.shortSlots = highWater;
+  p.numSlots = highWater + longCount;
   p.numInstructions = uint32_t(instrs.size());
   std::ostringstream hdr;
   hdr << "; interpreter program for SPN '" << g.name << "': " << instrs.size() << " instructions, " << p.code.size() << " words, "
-      << p.numSlots << " value slots (" << p.reservedSlots << " staged features), compute " << (p.f64 ? "f64" : "f32")
+      << p.numSlots << " value slots (" << p.reservedSlots << " staged features, " << (p.numSlots - p.shortSlots) << " long-lived), compute " << (p.f64 ? "f64" : "f32")
       << (p.log2Domain ? " log2-domain" : "") << ", features " << (p.featureMode == FEAT_STAGED ? "staged" : "direct") << "\n";
   p.listing = hdr.str() + b.txt.str();
   return p;
 }
+}  // namespace
 
 }  // namespace spnc_hip

@@ -13,12 +13,15 @@
 
 namespace spnc_hip {
 
-// Opcodes (low 8 bits of an instruction's first word; the upper 24 bits hold a count).
+// Opcodes (low 7 bits of an instruction's first word; bit 7 is set when the instruction reads or
+// writes a long-lived slot; the upper 24 bits hold counts).
 enum InterpOp : uint32_t {
   OP_END = 0,       // [op][src]                       result = slot src
-  OP_PROD = 1,      // [op][dst][ns][ng][nt] ns*slot, ng*(feat, mean, coef, den), nt*(feat, tableOffset)
+  OP_PROD = 1,      // [op][dst][ns][ng][nt] ns*slot, ng*(feat, mean, coef, den), nt*(feat, tableOffset, tableLen)
   OP_SUM = 2,       // [op|k<<8][dst] k*(slot, weight)                 one weighted sum
   OP_SUMLAYER = 3,  // [op|k<<8][M][dst*M] k*slot, k*M weights        M sums over the same k children (M in 2,4,8)
+  OP_OUTERSUM = 4,  // [op|NA<<8|NB<<16][M][dst*M] NA*slot, NB*slot, NA*NB*M weights
+                    //   M sums over all products a_r * b_c of two operand vectors, products never materialised
 };
 
 // How leaves obtain their feature value.
@@ -43,6 +46,7 @@ struct InterpProgram {
   std::vector<uint32_t> directTableLen;  // FEAT_DIRECT: per column clamp bound (0 = none)
   std::vector<StagedFeature> staged;
   uint32_t numSlots = 0;      // value slots the program addresses, staged features included
+  uint32_t shortSlots = 0;    // slots [0, shortSlots) are the busy ones; [shortSlots, numSlots) hold long-lived values
   uint32_t reservedSlots = 0; // leading slots pinned to staged features
   uint32_t numInstructions = 0;
   std::string listing;        // human-readable form, for "dump-ir"

@@ -154,6 +154,7 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
     k->blockSize_ = js.blockSize;
     k->samplesPerLane_ = js.samplesPerLane;
     k->inputAlign_ = js.inputAlign;
+    k->gridPolicy_ = o.blocksPerCU != 0 ? o.blocksPerCU : (js.oneTilePerBlock ? -1 : 0);
     k->bytesPerResult_ = js.bytesPerResult;
     k->text_ = std::move(js.source);
   }
@@ -192,6 +193,7 @@ void Kernel::save(const std::string& path) const {
     w.u32(blockSize_);
     w.u32(samplesPerLane_);
     w.u32(inputAlign_);
+    w.u32(uint32_t(gridPolicy_));
   } else {
     w.u32(prog_.f64);
     w.u32(prog_.log2Domain);
@@ -207,6 +209,7 @@ void Kernel::save(const std::string& path) const {
       w.u32(s.tableLen);
     }
     w.u32(prog_.numSlots);
+    w.u32(prog_.shortSlots);
     w.u32(prog_.reservedSlots);
     w.u32(prog_.numInstructions);
   }
@@ -243,6 +246,7 @@ std::unique_ptr<Kernel> Kernel::load(const std::string& kernelFile) {
     k->blockSize_ = r.u32();
     k->samplesPerLane_ = r.u32();
     k->inputAlign_ = r.u32();
+    k->gridPolicy_ = int(r.u32());
   } else if (k->kind_ == SPNC_HIP_KERNEL_INTERPRETER) {
     k->prog_.f64 = r.u32() != 0;
     k->prog_.log2Domain = r.u32() != 0;
@@ -260,6 +264,7 @@ std::unique_ptr<Kernel> Kernel::load(const std::string& kernelFile) {
       k->prog_.staged.push_back(s);
     }
     k->prog_.numSlots = r.u32();
+    k->prog_.shortSlots = r.u32();
     k->prog_.reservedSlots = r.u32();
     k->prog_.numInstructions = r.u32();
     k->inputAlign_ = k->bytesPerFeature_;
@@ -325,10 +330,19 @@ void Kernel::ensureDevice() {
     hipCheck(interpreterMaxLds(prog_.f64, prog_.log2Domain, &maxBlock), "LDS limit query");
     size_t budget = std::min<size_t>(maxBlock, size_t(ldsPerCU) / 2);
     uint32_t cap = uint32_t(budget / (INTERP_BLOCK * rb));
-    ldsSlots_ = std::min(prog_.numSlots, cap);
+    if (prog_.numSlots <= cap) {
+      ldsSlots_ = prog_.numSlots;
+      interpMode_ = 0;
+    } else if (prog_.shortSlots <= cap) {
+      ldsSlots_ = prog_.shortSlots;  // long-lived values go to the spill tier, only flagged instructions see them
+      interpMode_ = 1;
+    } else {
+      ldsSlots_ = cap;
+      interpMode_ = 2;
+    }
     ldsBytes_ = size_t(ldsSlots_) * INTERP_BLOCK * rb;
     int nb = 0;
-    hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, ldsBytes_, &nb), "occupancy query");
+    hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, interpMode_, ldsBytes_, &nb), "occupancy query");
     blocksPerCU_ = std::max(1, nb);
     hipCheck(hipMalloc(&dCode_, prog_.code.size() * 4), "hipMalloc(program)");
     hipCheck(hipMemcpy(dCode_, prog_.code.data(), prog_.code.size() * 4, hipMemcpyHostToDevice), "program upload");
@@ -394,7 +408,10 @@ void Kernel::launch(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
   if (kind_ == SPNC_HIP_KERNEL_JIT) {
     const size_t tile = size_t(blockSize_) * samplesPerLane_;
     const size_t tiles = (n + tile - 1) / tile;
-    const unsigned grid = unsigned(std::min<size_t>(tiles, size_t(numCUs_) * blocksPerCU_));
+    size_t cap = size_t(numCUs_) * blocksPerCU_;
+    if (gridPolicy_ < 0) cap = tiles;
+    else if (gridPolicy_ > 0) cap = size_t(numCUs_) * gridPolicy_;
+    const unsigned grid = unsigned(std::min<size_t>(std::min<size_t>(tiles, cap), 0x7fffffffu));
     unsigned long long n64 = n;
     void* args[] = {(void*)&dIn, (void*)&dOut, (void*)&n64};
     hipCheck(hipModuleLaunchKernel(function_, grid, 1, 1, blockSize_, 1, 1, 0, stream, args, nullptr), "kernel launch");
@@ -415,7 +432,7 @@ void Kernel::launch(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
     a.featureMode = prog_.featureMode;
     a.ldsSlots = ldsSlots_;
     a.marginal = marginal_ ? 1u : 0u;
-    hipCheck(launchInterpreter(a, prog_.f64, prog_.log2Domain, grid, ldsBytes_, stream), "interpreter launch");
+    hipCheck(launchInterpreter(a, prog_.f64, prog_.log2Domain, interpMode_, grid, ldsBytes_, stream), "interpreter launch");
   }
 }
 

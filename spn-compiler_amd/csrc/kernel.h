@@ -59,6 +59,7 @@ class Kernel {
   std::vector<char> codeObject_;
   std::string entry_;
   unsigned blockSize_ = 256, samplesPerLane_ = 1, inputAlign_ = 4;
+  int gridPolicy_ = 0;  // 0 = resident blocks, -1 = one tile per block, n = n blocks per CU
   // interpreter
   InterpProgram prog_;
 
@@ -76,6 +77,7 @@ class Kernel {
   void* dSpill_ = nullptr;
   size_t spillBytes_ = 0;
   uint32_t ldsSlots_ = 0;
+  int interpMode_ = 0;
   size_t ldsBytes_ = 0;
   // double-buffered staging for host execute
   struct Stage {

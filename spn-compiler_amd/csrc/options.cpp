@@ -50,7 +50,7 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
     } else if (key == "use-log-space") {
       o.useLogSpace = parseBool(val);
     } else if (key == "gpu-shared-mem") {
-      o.gpuSharedMem = parseBool(val);
+      o.gpuSharedMem = parseBool(val) ? 1 : 0;
     } else if (key == "dump-ir") {
       o.dumpIR = parseBool(val);
     } else if (key == "collect-graph-stats") {
@@ -83,6 +83,9 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       if (o.samplesPerLane < 0 || o.samplesPerLane > 16) throw std::runtime_error("hip-samples-per-lane must be in [0,16]");
     } else if (key == "hip-jit-max-ops") {
       o.jitMaxOps = parseInt(key, val);
+    } else if (key == "hip-blocks-per-cu") {
+      o.blocksPerCU = parseInt(key, val);
+      if (o.blocksPerCU < -1 || o.blocksPerCU > 64) throw std::runtime_error("hip-blocks-per-cu must be in [-1,64]");
     } else if (key == "hip-block-size") {
       o.blockSize = parseInt(key, val);
       if (o.blockSize != 64 && o.blockSize != 128 && o.blockSize != 256 && o.blockSize != 512)

@@ -16,7 +16,7 @@ enum class ComputeType { F32, F64 };
 
 struct CompileOptions {
   bool useLogSpace = false;     // "use-log-space" (reference default false; the Python front passes true)
-  bool gpuSharedMem = true;     // "gpu-shared-mem": stage the input tile through LDS
+  int gpuSharedMem = -1;        // "gpu-shared-mem": stage the input tile through LDS (1), do not (0), decide from the SPN (-1, option absent)
   bool dumpIR = false;          // "dump-ir": print the generated device source / program
   bool collectGraphStats = false;
   std::string graphStatsFile = "/tmp/stats.json";
@@ -30,6 +30,7 @@ struct CompileOptions {
   int samplesPerLane = 0;                      // "hip-samples-per-lane": 0 = choose from SPN size
   int jitMaxOps = 20000;                       // "hip-jit-max-ops": above this, auto picks the interpreter
   int blockSize = 256;                         // "hip-block-size"
+  int blocksPerCU = 0;                         // "hip-blocks-per-cu": 0 = resident blocks (persistent), -1 = one tile per block, n = n per CU
 };
 
 // Throws std::runtime_error("Unknown compile option <key>") etc.

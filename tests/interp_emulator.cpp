@@ -1,0 +1,144 @@
+// CPU emulation of an interpreter program, with bounds checks on every slot and code access.
+// Test aid: builds the program for a serialized query exactly as the library does, checks its
+// structural invariants (slot numbers in range, only flagged instructions touch the long-lived
+// pool) and evaluates it in float for rows of doubles read from a file, one result per line.
+//   usage: interp_emulator <query.bin> <inputs.f64> <rows> [key=value ...]
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../spn-compiler_amd/csrc/interp_program.h"
+#include "../spn-compiler_amd/csrc/options.h"
+#include "../spn-compiler_amd/csrc/spn_graph.h"
+using namespace spnc_hip;
+
+static float asFloat(uint32_t w) {
+  float f;
+  std::memcpy(&f, &w, 4);
+  return f;
+}
+
+int main(int argc, char** argv) {
+  if (argc < 4) return 2;
+  try {
+    Graph g = buildGraph(readQueryFile(argv[1]));
+    std::map<std::string, std::string> kv{{"target", "HIP"}, {"use-log-space", "true"}};
+    for (int i = 4; i < argc; ++i) {
+      std::string a = argv[i];
+      kv[a.substr(0, a.find('='))] = a.substr(a.find('=') + 1);
+    }
+    InterpProgram p = buildInterpProgram(g, parseOptions(kv));
+    if (p.f64) throw std::runtime_error("emulator evaluates float programs only");
+    const size_t rows = std::stoul(argv[3]);
+    std::vector<double> in(rows * g.numFeatures);
+    FILE* f = std::fopen(argv[2], "rb");
+    if (!f || std::fread(in.data(), 8, in.size(), f) != in.size()) throw std::runtime_error("cannot read inputs");
+    std::fclose(f);
+    std::fprintf(stderr, "instructions %u words %zu slots %u short %u reserved %u\n", p.numInstructions, p.code.size(), p.numSlots,
+                 p.shortSlots, p.reservedSlots);
+    const auto& c = p.code;
+    std::vector<float> tab(p.tables.begin(), p.tables.end());
+    const float finish = p.log2Domain ? 0.6931471805599453f : 1.0f;
+    auto ex = [&](float v) { return p.log2Domain ? std::exp2(v) : std::exp(v); };
+    auto lg = [&](float v) { return p.log2Domain ? std::log2(v) : std::log(v); };
+    for (size_t row = 0; row < rows; ++row) {
+      const double* x = &in[row * g.numFeatures];
+      std::vector<float> slot(p.numSlots, NAN);
+      auto index = [&](double v, uint32_t L) -> uint32_t {
+        if (v != v) return g.supportMarginal ? L + 1 : L;
+        return (v > -1.0 && v < double(L)) ? uint32_t(v) : L;
+      };
+      for (const auto& s : p.staged) {
+        if (s.valueSlot != UINT32_MAX) slot.at(s.valueSlot) = float(x[s.column]);
+        if (s.indexSlot != UINT32_MAX) slot.at(s.indexSlot) = float(index(x[s.column], s.tableLen));
+      }
+      size_t pc = 0;
+      for (;;) {
+        const uint32_t w0 = c.at(pc), op = w0 & 0x7f;
+        const bool flagged = w0 & 0x80;
+        auto rd = [&](uint32_t s) {
+          if (!flagged && s >= p.shortSlots) throw std::runtime_error("unflagged instruction reads long-lived slot at word " + std::to_string(pc));
+          return slot.at(s);
+        };
+        auto wr = [&](uint32_t s, float v) {
+          if (!flagged && s >= p.shortSlots) throw std::runtime_error("unflagged instruction writes long-lived slot at word " + std::to_string(pc));
+          slot.at(s) = v;
+        };
+        if (op == OP_END) {
+          std::printf("%.9g\n", rd(c.at(pc + 1)) * finish);
+          break;
+        }
+        if (op == OP_PROD) {
+          const uint32_t dst = c.at(pc + 1), ns = c.at(pc + 2), ng = c.at(pc + 3), nt = c.at(pc + 4);
+          size_t q = pc + 5;
+          float acc = 0;
+          for (uint32_t j = 0; j < ns; ++j) acc += rd(c.at(q + j));
+          q += ns;
+          for (uint32_t j = 0; j < ng; ++j, q += 4) {
+            const float xv = p.featureMode == FEAT_STAGED ? rd(c.at(q)) : float(x[c.at(q)]);
+            const float d = xv - asFloat(c.at(q + 1));
+            float v = asFloat(c.at(q + 2)) + d * d * asFloat(c.at(q + 3));
+            if (g.supportMarginal && xv != xv) v = 0;
+            acc += v;
+          }
+          for (uint32_t j = 0; j < nt; ++j, q += 3) {
+            const uint32_t idx = p.featureMode == FEAT_STAGED ? uint32_t(rd(c.at(q))) : index(x[c.at(q)], c.at(q + 2));
+            acc += tab.at(c.at(q + 1) + idx);
+          }
+          wr(dst, acc);
+          pc = q;
+        } else if (op == OP_SUM) {
+          const uint32_t k = w0 >> 8, dst = c.at(pc + 1);
+          size_t q = pc + 2;
+          if (k == 1) {
+            wr(dst, rd(c.at(q)) + asFloat(c.at(q + 1)));
+            pc = q + 2;
+            continue;
+          }
+          float m = -INFINITY, acc = 0;
+          for (uint32_t j = 0; j < k; ++j) m = std::fmax(m, rd(c.at(q + 2 * j)));
+          m = std::fmax(m, -3.4028234663852886e38f);
+          for (uint32_t j = 0; j < k; ++j) acc += ex(rd(c.at(q + 2 * j)) - m) * asFloat(c.at(q + 2 * j + 1));
+          wr(dst, m + lg(acc));
+          pc = q + 2 * k;
+        } else if (op == OP_SUMLAYER) {
+          const uint32_t k = w0 >> 8, M = c.at(pc + 1);
+          const size_t d0 = pc + 2, k0 = d0 + M, w = k0 + k;
+          float m = -INFINITY;
+          for (uint32_t j = 0; j < k; ++j) m = std::fmax(m, rd(c.at(k0 + j)));
+          m = std::fmax(m, -3.4028234663852886e38f);
+          std::vector<float> res(M, 0.f);
+          for (uint32_t t = 0; t < M; ++t)
+            for (uint32_t j = 0; j < k; ++j) res[t] += ex(rd(c.at(k0 + j)) - m) * asFloat(c.at(w + j * M + t));
+          for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), m + lg(res[t]));
+          pc = w + size_t(k) * M;
+        } else if (op == OP_OUTERSUM) {
+          const uint32_t na = (w0 >> 8) & 0xff, nb = w0 >> 16, M = c.at(pc + 1);
+          const size_t d0 = pc + 2, a0 = d0 + M, b0 = a0 + na, w = b0 + nb;
+          float ma = -INFINITY, mb = -INFINITY;
+          for (uint32_t r = 0; r < na; ++r) ma = std::fmax(ma, rd(c.at(a0 + r)));
+          for (uint32_t cc = 0; cc < nb; ++cc) mb = std::fmax(mb, rd(c.at(b0 + cc)));
+          ma = std::fmax(ma, -3.4028234663852886e38f);
+          mb = std::fmax(mb, -3.4028234663852886e38f);
+          std::vector<float> res(M, 0.f);
+          for (uint32_t t = 0; t < M; ++t)
+            for (uint32_t r = 0; r < na; ++r)
+              for (uint32_t cc = 0; cc < nb; ++cc)
+                res[t] += ex(rd(c.at(a0 + r)) - ma) * ex(rd(c.at(b0 + cc)) - mb) * asFloat(c.at(w + (size_t(r) * nb + cc) * M + t));
+          for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), ma + mb + lg(res[t]));
+          pc = w + size_t(na) * nb * M;
+        } else {
+          throw std::runtime_error("unknown opcode at word " + std::to_string(pc));
+        }
+      }
+    }
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "emulator error: %s\n", e.what());
+    return 1;
+  }
+  return 0;
+}
