@@ -352,7 +352,7 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
     if (stagedMode) {
       for (int s = 0; s < int(a.numStaged); ++s) {
         const uint32_t col = staged[4 * s], vs = staged[4 * s + 1], is = staged[4 * s + 2], L = staged[4 * s + 3];
-        if (MODE == 2) {
+        if (MODE != 0) {
           if (vs != NONE) Sg.wr(vs, featureValue<R>(a.in, a.featureType, row + col));
           if (is != NONE) Sg.wr(is, R(featureIndex(a.in, a.featureType, row + col, L, a.marginal)));
         } else {

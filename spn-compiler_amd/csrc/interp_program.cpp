@@ -42,31 +42,44 @@ struct Builder {
 }  // namespace
 
 namespace {
-InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t longRange);
+InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t longRange, bool stagedLong);
 }
 
 // Values that stay live for more than `longRange` instructions are numbered after all the others
 // ("long pool"), so that the launcher can keep the busy, short-lived slots in LDS and the rarely
-// touched long-lived ones in the spill tier. The range is lowered until the short pool fits the
-// LDS share that lets two blocks reside on a CU.
+// touched long-lived ones in the spill tier; the staged feature values can be moved there too.
+// Candidates are tried from "everything short" towards "as little as possible short" until the
+// short pool fits the LDS share that lets four blocks reside on a CU, or failing that two.
 InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
-  const uint32_t target = o.computeType == ComputeType::F64 ? 36 : 72;
+  const bool f64 = o.computeType == ComputeType::F64;
+  const uint32_t fourBlocks = f64 ? 20 : 40, twoBlocks = f64 ? 36 : 72;
   InterpProgram best;
   bool have = false;
-  for (uint32_t range : {0xffffffffu, 512u, 256u, 128u, 64u, 32u, 16u, 8u}) {
-    InterpProgram p = buildWithRange(g, o, range);
-    const bool fits = p.shortSlots <= target;
-    if (!have || p.shortSlots < best.shortSlots) {
-      best = std::move(p);
-      have = true;
+  auto better = [&](const InterpProgram& p) {
+    if (!have) return true;
+    const bool p4 = p.shortSlots <= fourBlocks, b4 = best.shortSlots <= fourBlocks;
+    const bool p2 = p.shortSlots <= twoBlocks, b2 = best.shortSlots <= twoBlocks;
+    if (p4 != b4) return p4;
+    if (p4) return false;  // the earlier candidate keeps more values in LDS
+    if (p2 != b2) return p2;
+    if (p2) return false;
+    return p.shortSlots < best.shortSlots;
+  };
+  for (bool stagedLong : {false, true}) {
+    for (uint32_t range : {0xffffffffu, 256u, 64u, 32u, 16u, 8u}) {
+      InterpProgram p = buildWithRange(g, o, range, stagedLong);
+      if (better(p)) {
+        best = std::move(p);
+        have = true;
+      }
+      if (best.shortSlots <= fourBlocks) return best;
     }
-    if (fits) break;
   }
   return best;
 }
 
 namespace {
-InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t longRange) {
+InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t longRange, bool stagedLong) {
   if (!o.useLogSpace) throw std::runtime_error("The interpreter kernel supports log-space computation only");
   InterpProgram p;
   p.f64 = o.computeType == ComputeType::F64;
@@ -101,19 +114,21 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   }
   p.featureMode = stagedSlots <= 48 ? FEAT_STAGED : FEAT_DIRECT;
   std::vector<uint32_t> valueSlotOf(g.numFeatures, NONE), indexSlotOf(g.numFeatures, NONE);
-  uint32_t nextSlot = 0;
+  constexpr uint32_t LONG_BIT = 0x80000000u;  // marks long-pool slot numbers until they are renumbered
+  uint32_t nextSlot = 0, longCount = 0;
+  auto stagedSlot = [&]() { return stagedLong ? (LONG_BIT | longCount++) : nextSlot++; };
   if (p.featureMode == FEAT_STAGED) {
     for (uint32_t f = 0; f < g.numFeatures; ++f) {
       if (!featGauss[f] && !featTableLen[f]) continue;
       StagedFeature sf{f, NONE, NONE, featTableLen[f]};
-      if (featGauss[f]) sf.valueSlot = valueSlotOf[f] = nextSlot++;
-      if (featTableLen[f]) sf.indexSlot = indexSlotOf[f] = nextSlot++;
+      if (featGauss[f]) sf.valueSlot = valueSlotOf[f] = stagedSlot();
+      if (featTableLen[f]) sf.indexSlot = indexSlotOf[f] = stagedSlot();
       p.staged.push_back(sf);
     }
   } else {
     p.directTableLen = featTableLen;
   }
-  p.reservedSlots = nextSlot;
+  p.reservedSlots = nextSlot + longCount;
 
   // ---- instruction selection ----
   // A leaf whose only consumer is a product is evaluated inside that product. Every other leaf
@@ -245,11 +260,10 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   std::vector<uint32_t> firstDef(N, 0);
   for (uint32_t k = 0; k < instrs.size(); ++k)
     for (uint32_t d : instrs[k].defs) firstDef[d] = k;
-  constexpr uint32_t LONG_BIT = 0x80000000u;  // marks long-pool slot numbers until they are renumbered
   std::vector<uint32_t> slotOf(N, NONE);
   typedef std::priority_queue<uint32_t, std::vector<uint32_t>, std::greater<uint32_t>> MinHeap;
   MinHeap freeShort, freeLong;
-  uint32_t highWater = nextSlot, longCount = 0;
+  uint32_t highWater = nextSlot;
   auto allocSlot = [&](uint32_t node) {
     const bool isLong = lastUse[node] - firstDef[node] > longRange;
     MinHeap& heap = isLong ? freeLong : freeShort;
@@ -273,12 +287,14 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
     if (leaf.kind == NodeKind::Gaussian) {
       double coef = -std::log(leaf.stddev) + -0.5 * std::log(2 * M_PI);
       double den = -(1.0 / (2.0 * leaf.stddev * leaf.stddev));
-      b.word(p.featureMode == FEAT_STAGED ? valueSlotOf[leaf.feature] : leaf.feature);
+      if (p.featureMode == FEAT_STAGED) slotWord(valueSlotOf[leaf.feature]);
+      else b.word(leaf.feature);
       b.real(leaf.mean);
       b.real(coef * b.scale);
       b.real(den * b.scale);
     } else {
-      b.word(p.featureMode == FEAT_STAGED ? indexSlotOf[leaf.feature] : leaf.feature);
+      if (p.featureMode == FEAT_STAGED) slotWord(indexSlotOf[leaf.feature]);
+      else b.word(leaf.feature);
       b.word(tableOffset[c]);
       b.word(featTableLen[leaf.feature]);
     }
@@ -310,6 +326,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
           for (uint32_t c : n.children)
             if (inlined[c]) (isTable(c) ? ts : gs).push_back(c);
         }
+        if (stagedLong && p.featureMode == FEAT_STAGED && !(gs.empty() && ts.empty())) longFlag |= 0x80u;
         b.word(OP_PROD | longFlag);
         slotWord(slotOf[in.node]);
         b.word(uint32_t(in.srcs.size()));
@@ -374,6 +391,10 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   b.word(OP_END | ((slotOf[g.root()] & LONG_BIT) ? 0x80u : 0u));
   slotWord(slotOf[g.root()]);
   for (size_t pos : longWords) p.code[pos] = highWater + (p.code[pos] & ~LONG_BIT);
+  for (auto& sf : p.staged) {
+    if (sf.valueSlot != NONE && (sf.valueSlot & LONG_BIT)) sf.valueSlot = highWater + (sf.valueSlot & ~LONG_BIT);
+    if (sf.indexSlot != NONE && (sf.indexSlot & LONG_BIT)) sf.indexSlot = highWater + (sf.indexSlot & ~LONG_BIT);
+  }
   p.shortSlots = highWater;
   p.numSlots = highWater + longCount;
   p.numInstructions = uint32_t(instrs.size());
