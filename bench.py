@@ -116,6 +116,16 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None):
         "valu_issue_frac": round(t_min_valu / t_launch, 4),
         "hbm_frac": round(t_min_hbm / t_launch, 4),
     }
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by what a
+    # plain copy of known size reads on the same counters); recorded per workload under profiles/.
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            entry = json.load(f).get(name)
+        if entry and entry.get("samples") == n:
+            roof["traffic"] = entry["bytes_per_launch"]
+            roof["traffic_over_algorithmic"] = round(entry["bytes_per_launch"] / (bytes_per_sample * n), 3)
+    except (OSError, ValueError):
+        pass
     res = {
         "workload": name, "desc": cfg["desc"], "n": n, "samples_per_s": n * steps / wall, "ms_per_step": wall / steps * 1e3,
         "roofline": roof, "compile_s": round(compile_s, 2), "nodes": info["num_nodes"], "finite": finite,

@@ -21,7 +21,8 @@ struct Emitter {
   double scale;  // multiplies natural-log constants (log2(e) in the log2 domain)
   std::ostringstream body;
   std::vector<double> tablePool;
-  std::vector<uint32_t> tableOffset;   // per node
+  std::vector<uint32_t> tableOffset;   // per node (for a paired leaf: offset of the joint table, held by the first of the pair)
+  std::vector<uint32_t> partner;       // per node: the table leaf it shares a joint table with, or UINT32_MAX
   std::vector<uint32_t> featTableLen;  // per feature: longest table of any leaf on it (0 = none)
   std::vector<bool> featGauss;         // per feature: used by a Gaussian leaf
   std::vector<bool> featUsed;
@@ -93,20 +94,72 @@ struct Emitter {
         featUsed[n.feature] = true;
       }
     }
-    // Table pool: every table leaf on feature f owns L_f + 2 entries: its own values, then
-    // "impossible" (log 0 / 0) up to index L_f for out-of-range inputs, then the marginal
-    // value (log 1 / 1) at L_f + 1 for NaN inputs. The index is clamped once per feature.
+    // Table pool: every table leaf on feature f owns L_f + 1 entries, its own values and then
+    // "impossible" (log 0 / 0) up to index L_f for out-of-range inputs, plus, when the query
+    // supports marginalisation, the marginal value (log 1 / 1) at L_f + 1 for NaN inputs.
+    // The index is clamped once per feature.
     tableOffset.assign(g.nodes.size(), 0);
-    for (size_t i = 0; i < g.nodes.size(); ++i) {
-      const auto& n = g.nodes[i];
-      if (n.kind != NodeKind::Categorical && n.kind != NodeKind::Histogram) continue;
-      uint32_t L = featTableLen[n.feature];
-      tableOffset[i] = uint32_t(tablePool.size());
+    partner.assign(g.nodes.size(), UINT32_MAX);
+    auto isTable = [&](uint32_t c) { return g.nodes[c].kind == NodeKind::Categorical || g.nodes[c].kind == NodeKind::Histogram; };
+    auto padded = [&](uint32_t c) {
+      const auto& n = g.nodes[c];
+      const uint32_t L = featTableLen[n.feature];
+      std::vector<double> t;
       for (uint32_t j = 0; j <= L; ++j) {
         double p = j < n.table.size() ? n.table[j] : 0.0;
-        tablePool.push_back(logSpace ? logConst(p) : p);
+        t.push_back(logSpace ? logConst(p) : p);
       }
-      tablePool.push_back(logSpace ? 0.0 : 1.0);
+      if (g.supportMarginal) t.push_back(logSpace ? 0.0 : 1.0);
+      return t;
+    };
+    auto rowLen = [&](uint32_t feature) { return size_t(featTableLen[feature]) + (g.supportMarginal ? 2 : 1); };
+    // Joint tables: two table leaves read only by the same product are replaced by one table over
+    // the pair of indices, J[i][j] = T_a[i] (+ or *) T_b[j], combined in double. One LDS read and one
+    // integer multiply-add then stand in for two LDS reads and one add; LDS reads are what bounds
+    // table-heavy SPNs. Pairing stops when the pool would outgrow its LDS budget.
+    const size_t realBytes = f64 ? 8 : 4, budget = 62 * 1024;  // LDS instruction offsets reach 64 KiB
+    size_t plain = 0;
+    for (uint32_t i = 0; i < g.nodes.size(); ++i)
+      if (isTable(i)) plain += rowLen(g.nodes[i].feature);
+    // Candidates: within a product, leaves ordered by table length and paired neighbour with
+    // neighbour (small with small); globally the cheapest pairs are taken first.
+    struct Candidate {
+      size_t extra;
+      uint32_t a, b;
+    };
+    std::vector<Candidate> candidates;
+    for (uint32_t i = 0; i < g.nodes.size() && o.jointTables; ++i) {
+      if (g.nodes[i].kind != NodeKind::Product) continue;
+      std::vector<uint32_t> leaves;
+      for (uint32_t c : g.nodes[i].children)
+        if (isTable(c) && g.nodes[c].uses == 1) leaves.push_back(c);
+      std::stable_sort(leaves.begin(), leaves.end(),
+                       [&](uint32_t x, uint32_t y) { return rowLen(g.nodes[x].feature) < rowLen(g.nodes[y].feature); });
+      for (size_t k = 0; k + 1 < leaves.size(); k += 2) {
+        const size_t ra = rowLen(g.nodes[leaves[k]].feature), rb = rowLen(g.nodes[leaves[k + 1]].feature);
+        if (ra * rb <= 160) candidates.push_back({ra * rb - ra - rb, leaves[k], leaves[k + 1]});
+      }
+    }
+    std::stable_sort(candidates.begin(), candidates.end(), [](const Candidate& x, const Candidate& y) { return x.extra < y.extra; });
+    size_t projected = plain;
+    for (const Candidate& c : candidates) {
+      if ((projected + c.extra) * realBytes > budget) break;
+      projected += c.extra;
+      partner[c.a] = c.b;
+      partner[c.b] = c.a;
+    }
+    for (uint32_t i = 0; i < g.nodes.size(); ++i) {
+      if (!isTable(i)) continue;
+      if (partner[i] != UINT32_MAX && partner[i] < i) continue;  // second leaf of a pair: lives in the joint table
+      tableOffset[i] = uint32_t(tablePool.size());
+      std::vector<double> a = padded(i);
+      if (partner[i] == UINT32_MAX) {
+        tablePool.insert(tablePool.end(), a.begin(), a.end());
+      } else {
+        std::vector<double> b = padded(partner[i]);
+        for (double x : a)
+          for (double y : b) tablePool.push_back(logSpace ? x + y : x * y);
+      }
     }
   }
 
@@ -167,6 +220,31 @@ struct Emitter {
     return false;
   }
 
+  // Names of the values a product combines, emitting whatever is not there yet. Two table
+  // leaves that share a joint table count as one operand.
+  std::vector<std::string> productOperands(const std::vector<uint32_t>& kids) {
+    std::vector<std::string> ops;
+    for (uint32_t c : kids) {
+      const bool table = g.nodes[c].kind == NodeKind::Categorical || g.nodes[c].kind == NodeKind::Histogram;
+      if (!table || partner[c] == UINT32_MAX) {
+        emitNode(c);
+        ops.push_back(v(c));
+        continue;
+      }
+      const uint32_t a = std::min(c, partner[c]), b = std::max(c, partner[c]);
+      if (c != a) continue;  // the pair was emitted with its first leaf
+      const uint32_t fa = g.nodes[a].feature, fb = g.nodes[b].feature;
+      emitFeaturePrep(fa);
+      emitFeaturePrep(fb);
+      emitted[a] = emitted[b] = true;
+      const std::string name = "j" + std::to_string(a);
+      body << "  const real_t " << name << " = tab[" << tableOffset[a] << "u + t" << fa << " * " << (featTableLen[fb] + (g.supportMarginal ? 2 : 1))
+           << "u + t" << fb << "];\n";
+      ops.push_back(name);
+    }
+    return ops;
+  }
+
   // Log-space product with Gaussian leaves folded in. A leaf's value coef + d*d*den (d = x - mean)
   // is rewritten den * (d*d + coef/den), so that leaf plus accumulation cost three instructions
   // whose constants are all literals: d = x - mean; t = fma(d, d, coef/den); acc = fma(t, den, acc).
@@ -182,12 +260,9 @@ struct Emitter {
     std::string p = "p" + std::to_string(i) + "_";
     std::string acc;
     if (!rest.empty()) {
+      const std::vector<std::string> ops = productOperands(rest);
       std::string e = tree(
-          0, rest.size(),
-          [&](size_t k) {
-            emitNode(rest[k]);
-            return v(rest[k]);
-          },
+          0, ops.size(), [&](size_t k) { return ops[k]; },
           [&](const std::string& a, const std::string& b) { return "(" + a + " + " + b + ")"; });
       acc = p + "r";
       body << "  const real_t " << acc << " = " << e << ";\n";
@@ -248,12 +323,9 @@ struct Emitter {
           break;
         }
         const char* op = logSpace ? " + " : " * ";
+        const std::vector<std::string> ops = productOperands(n.children);
         std::string e = tree(
-            0, n.children.size(),
-            [&](size_t k) {
-              emitNode(n.children[k]);
-              return v(n.children[k]);
-            },
+            0, ops.size(), [&](size_t k) { return ops[k]; },
             [&](const std::string& a, const std::string& b) { return "(" + a + op + b + ")"; });
         body << "  const real_t " << v(i) << " = " << e << ";\n";
         break;
@@ -439,7 +511,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   else s << "  return " << root << ";\n";
   s << "}\n";
 
-  s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK) " << js.entry
+  s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK" << (o.minBlocksPerCU > 0 ? ", " + std::to_string(o.minBlocksPerCU) : std::string()) << ") " << js.entry
     << "(const feat_t* __restrict__ in, real_t* __restrict__ out, unsigned long long n) {\n";
   if (js.tableEntries && js.tablesInLds) {
     s << "  __shared__ real_t tab[SPN_NTAB];\n"

@@ -83,6 +83,11 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       if (o.samplesPerLane < 0 || o.samplesPerLane > 16) throw std::runtime_error("hip-samples-per-lane must be in [0,16]");
     } else if (key == "hip-jit-max-ops") {
       o.jitMaxOps = parseInt(key, val);
+    } else if (key == "hip-joint-tables") {
+      o.jointTables = parseBool(val);
+    } else if (key == "hip-min-blocks-per-cu") {
+      o.minBlocksPerCU = parseInt(key, val);
+      if (o.minBlocksPerCU < 0 || o.minBlocksPerCU > 8) throw std::runtime_error("hip-min-blocks-per-cu must be in [0,8]");
     } else if (key == "hip-blocks-per-cu") {
       o.blocksPerCU = parseInt(key, val);
       if (o.blocksPerCU < -1 || o.blocksPerCU > 64) throw std::runtime_error("hip-blocks-per-cu must be in [-1,64]");

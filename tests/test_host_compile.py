@@ -155,11 +155,14 @@ def test_scope_values_map_to_columns_in_ascending_order(native, tmp_path):
     # scope values {5, 2}: column 0 is scope 2, column 1 is scope 5
     path = rf.write(str(tmp_path / "s.bin"), nodes=[rf.cat(1, 5, p=(0.9, 0.1)), rf.cat(2, 2, p=(0.2, 0.8)), rf.prod(0, [1, 2])],
                     scope=[5, 2], feature_type="int32")
-    k = compile_query(native, path)
+    k = compile_query(native, path, **{"hip-joint-tables": "false"})
     src = k.source()
     first = src.index("tab[0u + t1]")   # first table (scope 5) is indexed by column 1
     second = src.index("u + t0]")       # second table (scope 2) by column 0
     assert first < second
+    os.remove(k.fileName())
+    k = compile_query(native, path)      # default: the two leaves of the product share one joint table, rows of 2 + 1 entries
+    assert "tab[0u + t1 * 3u + t0]" in k.source()
     os.remove(k.fileName())
 
 
