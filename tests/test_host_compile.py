@@ -186,7 +186,7 @@ def test_generated_source_variants(native):
     assert k.info()["kernel_kind"] == 2 and "sumlayer" not in k.source() and "sum(4 terms)" in k.source()
     os.remove(k.fileName())
     k = compile_spn(native, syn.c4_spn(), "float32")
-    assert k.info()["kernel_kind"] == 2 and "sumlayer(8 sums x 64 terms)" in k.source()
+    assert k.info()["kernel_kind"] == 2 and "outersum(8 sums x 8x8 products)" in k.source()
     os.remove(k.fileName())
 
 
