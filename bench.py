@@ -21,6 +21,7 @@ sys.path.insert(0, os.path.join(ROOT, "spn-compiler_amd"))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X FP32 vector, published
+FP64_VECTOR_PEAK_TFLOPS = 78.6   # MI355X FP64 vector, published
 
 
 def make_inputs(name, cfg, n, torch, device):
@@ -47,6 +48,8 @@ def make_inputs(name, cfg, n, torch, device):
 def measure(name, n, steps, warmup, torch, device, extra_options=None):
     from spnc import synthetic as syn
     from spnc.hip import HIPCompiler
+    if name == "c5_f64":   # configuration 5 computed in float64 log-space
+        name, extra_options = "c5", dict(extra_options or {}, **{"hip-compute-type": "float64"})
     cfg = syn.CONFIGS[name]
     n = n or cfg["n"]
     spn = cfg["spn"]()
@@ -84,7 +87,8 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None):
     # FP32 VALU issue rate: 128 lane-operations per CU per clock (a wave64 instruction issues in
     # two cycles on each of the four SIMDs). This is what the published 157.3 TFLOP/s is made of
     # (256 CUs x 128 lanes x 2 flops per FMA x 2.4 GHz); a transcendental takes four such slots.
-    valu_peak = props.multi_processor_count * 128 * clock_hz  # lane-operations per second
+    f64 = info["dtype"] == "float64"
+    valu_peak = props.multi_processor_count * (64 if f64 else 128) * clock_hz  # lane-operations per second
     t_launch = launch_ms * 1e-3
     hbm_gbs = bytes_per_sample * n / t_launch / 1e9
     tflops = flops * n / t_launch / 1e12
@@ -94,17 +98,18 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None):
     # Compute-bound kernels are priced in issue slots (simple op 1, transcendental 4) against the
     # FP32 vector peak for single-flop instructions, i.e. half the published FMA figure.
     slot_tflops = slots * n / t_launch / 1e12
-    slot_peak = FP32_VECTOR_PEAK_TFLOPS / 2
+    slot_peak = (FP64_VECTOR_PEAK_TFLOPS if f64 else FP32_VECTOR_PEAK_TFLOPS) / 2
     roof = {
-        "bound": "hbm" if hbm_bound else "valu-fp32",
+        "bound": "hbm" if hbm_bound else ("valu-fp64" if f64 else "valu-fp32"),
         "achieved": round(hbm_gbs if hbm_bound else slot_tflops, 3),
         "peak": HBM_PEAK_GBS if hbm_bound else slot_peak,
         "unit": "GB/s" if hbm_bound else "TFLOP/s",
         "frac": round((hbm_gbs / HBM_PEAK_GBS) if hbm_bound else (slot_tflops / slot_peak), 4),
         "traffic": None,
         "peak_note": ("published HBM3E bandwidth" if hbm_bound else
-                      "published FP32 vector peak 157.3 TFLOP/s counts an FMA as 2 flops; this path issues single-flop "
-                      "instructions, so the ceiling is 78.65 T issue slots/s; achieved = (flops + 3*transcendentals) per sample"),
+                      "published vector peak (FP32 157.3, FP64 78.6 TFLOP/s) counts an FMA as 2 flops; this path issues "
+                      "single-flop instructions, so the ceiling is half of it in issue slots/s; achieved = (flops + "
+                      "3*transcendentals) per sample; a float64 exp/log is in fact ~22 instructions, not 4 slots"),
         "fma_flops_tflops": round(tflops, 3),
         "kernel": "spn_kernel (hipRTC straight-line)" if info["kernel_kind"] == 1 else "spn_interp_kernel",
         "launch_ms": round(launch_ms, 4),
@@ -178,7 +183,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "c5_f64"])
     ap.add_argument("--n", type=int, default=0, help="override the number of samples")
     ap.add_argument("--no-others", action="store_true", help="measure only the selected configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -224,7 +229,7 @@ def main():
     torch.cuda.empty_cache()
     others = {}
     if not args.no_others:
-        for name in ["c1", "c2", "c3", "c4", "c5"]:
+        for name in ["c1", "c2", "c3", "c4", "c5", "c5_f64"]:
             if name == args.config:
                 continue
             with contextlib.redirect_stdout(log):

@@ -450,6 +450,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   if (U == 0) U = (work <= 4000 && !g.supportMarginal && size_t(js.tableEntries) * realBytes <= 16 * 1024) ? 2 : 1;
   if (!e.vectorRows) U = 1;
   js.samplesPerLane = U;
+  js.libraryMath = !e.log2Dom;
 
   std::ostringstream s;
   s << "// generated by spnc-hip for SPN '" << g.name << "': " << g.nodes.size() << " nodes, " << F << " features\n";

@@ -149,7 +149,12 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
   } else {
     k->kind_ = SPNC_HIP_KERNEL_JIT;
     JitSource js = emitHipSource(g, o);
-    k->codeObject_ = compileWithHipRtc(js, o.optLevel);
+    // The generated code is already straight-line and CSE'd. Kernels that inline the library
+    // exp/log are built at -O1 unless the caller asks otherwise: at -O2 and above the mid-level
+    // optimiser stretches live ranges until the float64 kernels spill (512 VGPRs plus scratch,
+    // about 7x slower on the 16-feature Gaussian tree).
+    const int level = (js.libraryMath && !o.optLevelGiven) ? 1 : o.optLevel;
+    k->codeObject_ = compileWithHipRtc(js, level);
     k->entry_ = js.entry;
     k->blockSize_ = js.blockSize;
     k->samplesPerLane_ = js.samplesPerLane;

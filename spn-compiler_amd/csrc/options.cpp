@@ -61,6 +61,7 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       o.maxTaskSize = parseInt(key, val);
     } else if (key == "optLevel") {
       o.optLevel = parseInt(key, val);
+      o.optLevelGiven = true;
     } else if (key == "delete-temps") {
       o.deleteTemps = parseBool(val);
     } else if (key == "hip-compute-type") {

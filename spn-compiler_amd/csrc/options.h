@@ -22,6 +22,7 @@ struct CompileOptions {
   std::string graphStatsFile = "/tmp/stats.json";
   int maxTaskSize = -1;
   int optLevel = 3;
+  bool optLevelGiven = false;   // "optLevel" was passed explicitly
   bool deleteTemps = true;
   ComputeType computeType = ComputeType::F32;  // "hip-compute-type": float32 | float64 (log-space only)
   KernelMode kernelMode = KernelMode::Auto;    // "hip-kernel": auto | jit | interpreter
