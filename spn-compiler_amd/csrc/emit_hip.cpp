@@ -172,7 +172,7 @@ struct Emitter {
       featPrepared[f] = true;
       std::string x = "x[" + std::to_string(f) + "]";
       if (!vectorRows) {
-        body << "  const feat_t x" << f << " = __builtin_nontemporal_load(row + " << f << ");\n";
+        body << "  const feat_t x" << f << " = SPN_LOAD(row + " << f << ");\n";
         x = "x" + std::to_string(f);
       }
       if (featGauss[f]) body << "  const real_t g" << f << " = (real_t)" << x << ";\n";
@@ -455,6 +455,12 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   std::ostringstream s;
   s << "// generated by spnc-hip for SPN '" << g.name << "': " << g.nodes.size() << " nodes, " << F << " features\n";
   s << "typedef " << (e.f64 ? "double" : "float") << " real_t;\n";
+  // Streaming (non-temporal) loads suit rows that one or two instructions per lane fetch whole and
+  // the coalesced tile copy; a wider row is fetched by many instructions per lane that revisit the
+  // same cache lines, which plain cached loads serve better (measured: +17 % on 400-byte rows).
+  const bool streaming = o.nontemporalLoads && g.numFeatures * g.ftype.bytes <= 32;
+  s << (streaming ? "#define SPN_LOAD(p) __builtin_nontemporal_load(p)\n" : "#define SPN_LOAD(p) (*(p))\n");
+  s << (o.nontemporalLoads ? "#define SPN_LOAD_TILE(p) __builtin_nontemporal_load(p)\n" : "#define SPN_LOAD_TILE(p) (*(p))\n");
   s << "typedef " << g.ftype.hipName << " feat_t;\n";
   if (vw > 1) s << "typedef feat_t rowvec_t __attribute__((ext_vector_type(" << vw << ")));\n";
   s << "#define SPN_F " << F << "\n#define SPN_BLOCK " << js.blockSize << "\n#define SPN_U " << U << "\n";
@@ -485,7 +491,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     if (vw == 1) {
       s << "  const feat_t* p = in + i * SPN_F;\n";
       for (unsigned f = 0; f < F; ++f)
-        if (e.featUsed[f]) s << "  x[" << f << "] = __builtin_nontemporal_load(p + " << f << ");\n";
+        if (e.featUsed[f]) s << "  x[" << f << "] = SPN_LOAD(p + " << f << ");\n";
     } else {
       s << "  const rowvec_t* p = reinterpret_cast<const rowvec_t*>(in + i * SPN_F);\n";
     }
@@ -493,13 +499,18 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
       bool used = false;
       for (unsigned k = 0; k < vw; ++k) used = used || e.featUsed[c * vw + k];
       if (!used) continue;
-      s << "  const rowvec_t r" << c << " = __builtin_nontemporal_load(p + " << c << ");\n";
+      s << "  const rowvec_t r" << c << " = SPN_LOAD(p + " << c << ");\n";
       for (unsigned k = 0; k < vw; ++k)
         if (e.featUsed[c * vw + k]) s << "  x[" << c * vw + k << "] = r" << c << "[" << k << "];\n";
     }
     s << "}\n";
   }
 
+  // Rows held in registers: derive the clamped table indices right away, so that a raw feature
+  // value and its index are never live together for long.
+  if (e.vectorRows && o.eagerIndices)
+    for (uint32_t f = 0; f < F; ++f)
+      if (e.featUsed[f] && e.featTableLen[f]) e.emitFeaturePrep(f);
   e.emitNode(g.root());
   if (e.vectorRows)
     s << "static __device__ __forceinline__ real_t spn_eval(const feat_t (&x)[SPN_F], const real_t* __restrict__ tab) {\n";
@@ -512,7 +523,16 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   else s << "  return " << root << ";\n";
   s << "}\n";
 
-  s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK" << (o.minBlocksPerCU > 0 ? ", " + std::to_string(o.minBlocksPerCU) : std::string()) << ") " << js.entry
+  // Large LDS tables leave room for two blocks per CU at most. The compiler is told to budget
+  // registers for two (256 VGPRs) when the indices held per lane leave enough of them for the
+  // arithmetic: two waves per SIMD issue VALU work at twice the rate of one and cover each
+  // other's LDS waits (C3: 4.6e9 -> 6.6e9 samples/s).
+  const size_t ldsTables = js.tablesInLds ? size_t(js.tableEntries) * realBytes : 0;
+  unsigned tableFeatures = 0;
+  for (uint32_t f = 0; f < F; ++f) tableFeatures += e.featTableLen[f] ? 1 : 0;
+  int minBlocks = o.minBlocksPerCU;
+  if (minBlocks == 0 && js.tablesInLds && ldsTables > 40 * 1024 && ldsTables <= 80 * 1024 && tableFeatures <= 136) minBlocks = 2;
+  s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK" << (minBlocks > 0 ? ", " + std::to_string(minBlocks) : std::string()) << ") " << js.entry
     << "(const feat_t* __restrict__ in, real_t* __restrict__ out, unsigned long long n) {\n";
   if (js.tableEntries && js.tablesInLds) {
     s << "  __shared__ real_t tab[SPN_NTAB];\n"
@@ -528,7 +548,6 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   // shared-memory preload (mlir/lib/Dialect/LoSPN/Passes/LoSPNGPUSharedMemoryInsertion.cpp:99-260)
   // and, like there, skipped when the tile does not fit.
   const size_t tileBytes = size_t(js.blockSize) * U * rowBytes;
-  const size_t ldsTables = js.tablesInLds ? size_t(js.tableEntries) * realBytes : 0;
   // Without an explicit option the tile is staged when the kernel is closer to the HBM bound
   // than to the VALU bound (about 6.4e12 B/s against 6e13 lane-operations/s on MI355X).
   const double tHbm = double(rowBytes + realBytes) / 6.4e12, tValu = double(g.stats.issueSlotsMin()) / 6.0e13;
@@ -558,7 +577,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
          "      spn_v4* dst = reinterpret_cast<spn_v4*>(spn_tile);\n"
          "      constexpr unsigned NV = SPN_BLOCK * SPN_U * SPN_F * sizeof(feat_t) / 16;\n"
          "#pragma unroll\n"
-         "      for (unsigned v = threadIdx.x; v < NV; v += SPN_BLOCK) dst[v] = __builtin_nontemporal_load(src + v);\n"
+         "      for (unsigned v = threadIdx.x; v < NV; v += SPN_BLOCK) dst[v] = SPN_LOAD_TILE(src + v);\n"
          "      __syncthreads();\n"
          "      feat_t x[SPN_U][SPN_F];\n"
          "#pragma unroll\n"

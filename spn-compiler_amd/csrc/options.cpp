@@ -84,6 +84,10 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       if (o.samplesPerLane < 0 || o.samplesPerLane > 16) throw std::runtime_error("hip-samples-per-lane must be in [0,16]");
     } else if (key == "hip-jit-max-ops") {
       o.jitMaxOps = parseInt(key, val);
+    } else if (key == "hip-nontemporal-loads") {
+      o.nontemporalLoads = parseBool(val);
+    } else if (key == "hip-eager-indices") {
+      o.eagerIndices = parseBool(val);
     } else if (key == "hip-joint-tables") {
       o.jointTables = parseBool(val);
     } else if (key == "hip-min-blocks-per-cu") {

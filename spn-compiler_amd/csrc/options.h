@@ -31,6 +31,8 @@ struct CompileOptions {
   int samplesPerLane = 0;                      // "hip-samples-per-lane": 0 = choose from SPN size
   int jitMaxOps = 20000;                       // "hip-jit-max-ops": above this, auto picks the interpreter
   int blockSize = 256;                         // "hip-block-size"
+  bool nontemporalLoads = true;                // "hip-nontemporal-loads": mark input loads as streaming
+  bool eagerIndices = true;                    // "hip-eager-indices": compute table indices of all features first
   bool jointTables = true;                     // "hip-joint-tables": pair table leaves of a product into joint tables
   int minBlocksPerCU = 0;                      // "hip-min-blocks-per-cu": register budget hint for the generated kernel (0 = none)
   int blocksPerCU = 0;                         // "hip-blocks-per-cu": 0 = resident blocks (persistent), -1 = one tile per block, n = n per CU
