@@ -371,7 +371,8 @@ struct Emitter {
       return fresh(v(c) + " + " + lit(w));
     };
     if (k == 1) {
-      body << "  const real_t " << v(i) << " = " << term(0) << ";\n";
+      const std::string only = term(0);  // emits the child first
+      body << "  const real_t " << v(i) << " = " << only << ";\n";
       return;
     }
     if (o.sumForm == SumForm::Pairwise) {

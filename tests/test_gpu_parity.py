@@ -314,3 +314,75 @@ def test_full_size_batches_repeat_a_checked_block(native, cfg, opts):
     assert np.abs(out[:block].cpu().numpy() - want).max() <= F32_TOL
     assert bool((out == out[:block][idx]).all())
     os.remove(k.fileName())
+
+
+# ---- randomly generated SPNs: DAGs with shared sub-graphs, mixed leaf kinds, uneven fan-in ----
+
+def _random_spn(seed, num_features, marginal):
+    from spnc.structure import Categorical, Gaussian, Histogram, Product, Sum
+    rng = np.random.default_rng(seed)
+    kinds = rng.integers(0, 3, num_features)        # per feature: 0 Gaussian, 1 Categorical, 2 Histogram
+    domains = rng.integers(2, 7, num_features)
+    pool = {}                                        # scope -> already built sub-SPNs, reused to make the graph a DAG
+
+    def leaf(f):
+        if kinds[f] == 0:
+            return Gaussian(float(rng.normal()), float(rng.uniform(0.2, 2.0)), scope=int(f))
+        p = rng.dirichlet(np.ones(domains[f]))
+        if rng.random() < 0.2:
+            p[rng.integers(0, len(p))] = 0.0         # an impossible category / empty bin
+            p = p / p.sum()
+        if kinds[f] == 1:
+            return Categorical(p=[float(v) for v in p], scope=int(f))
+        return Histogram(breaks=list(range(len(p) + 1)), densities=[float(v) for v in p], bin_repr_points=[0.5] * len(p), scope=int(f))
+
+    def build(scope, depth):
+        key = tuple(scope)
+        if key in pool and rng.random() < 0.4:
+            return pool[key][rng.integers(0, len(pool[key]))]
+        if len(scope) == 1:
+            node = leaf(scope[0])
+        elif depth >= 4 or rng.random() < 0.3:
+            node = Product(children=[leaf(f) for f in scope])
+        elif rng.random() < 0.5:
+            k = int(rng.integers(1, 20 if depth == 0 else 6))
+            node = Sum(weights=[float(w) for w in rng.dirichlet(np.ones(k))], children=[build(scope, depth + 1) for _ in range(k)])
+        else:
+            parts = int(rng.integers(2, min(4, len(scope)) + 1))
+            perm = [scope[i] for i in rng.permutation(len(scope))]
+            node = Product(children=[build(sorted(int(v) for v in part), depth + 1) for part in np.array_split(np.array(perm), parts)])
+        pool.setdefault(key, []).append(node)
+        return node
+
+    spn = build(list(range(num_features)), 0)
+    n = 257
+    X = np.empty((n, num_features), dtype=np.float64)
+    for f in range(num_features):
+        X[:, f] = rng.normal(0, 1.5, n) if kinds[f] == 0 else rng.integers(-1, domains[f] + 2, n)
+    if marginal:
+        X[rng.random(X.shape) < 0.15] = np.nan
+    return spn, X
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_spns(native, seed):
+    marginal = seed % 2 == 0
+    spn, X = _random_spn(1000 + seed, num_features=3 + seed, marginal=marginal)
+    m = oracle_model(spn, "float64")
+    want64 = ev.ll_closed_f64(m, X, marginal=marginal)
+    for opts in ({}, {"hip-kernel": "interpreter"}, {"hip-sum-form": "pairwise"}, {"hip-compute-type": "float64"},
+                 {"hip-compute-type": "float64", "hip-kernel": "interpreter"}):
+        got = run(compile_spn(native, spn, "float64", marginal=marginal, **opts), X)
+        finite = np.isfinite(want64)
+        if opts.get("hip-sum-form") != "pairwise":      # the pairwise tree turns (-inf) + (-inf) into NaN, like the reference
+            assert np.array_equal(np.isneginf(got), np.isneginf(want64)), opts
+        ok = finite & np.isfinite(got)
+        assert ok.sum() >= finite.sum() * 0.5
+        tol = F64_TOL if got.dtype == np.float64 else F32_TOL
+        assert np.abs(got[ok] - want64[ok]).max(initial=0) <= tol * max(1.0, np.abs(want64[ok]).max(initial=0) / 100 if got.dtype == np.float32 else 1.0), opts
+    if not marginal:                                    # integer inputs of the same values (negative ones wrap to huge unsigned: impossible)
+        Xi = np.where(np.isnan(X), 0, X).astype(np.int32)
+        has_gauss = any(n.kind == sm.GAUSSIAN for n in m.nodes)
+        if not has_gauss:
+            got = run(compile_spn(native, spn, "int32", **{}), Xi)
+            check_f32(got, oracle_model(spn, "int32"), Xi.astype(np.uint32), False)
