@@ -225,14 +225,32 @@ __device__ __forceinline__ code_ptr outerSumFixed(code_ptr ip, const Slots<R, fa
   R acc[M];
 #pragma unroll
   for (int t = 0; t < M; ++t) acc[t] = R(0);
+  // The weights arrive through scalar loads, whose wait counter is all-or-nothing: they are
+  // requested two chunks of PAIRS (r,c) pairs ahead and the scheduler is kept from moving the
+  // requests, so that two chunks of multiply-adds (and the other waves of the SIMD) cover the
+  // latency of a chunk's loads.
+  constexpr int PAIRS = (16 / RW) / M >= 1 ? (16 / RW) / M : 1, CHUNKS = NA * NB / PAIRS, AHEAD = 2;
+  static_assert(NA * NB % PAIRS == 0, "chunking must divide the weight matrix");
+  R wc[AHEAD + 1][PAIRS * M];
 #pragma unroll
-  for (int r = 0; r < NA; ++r) {
+  for (int q = 0; q < AHEAD && q < CHUNKS; ++q)
 #pragma unroll
-    for (int c = 0; c < NB; ++c) {
-      const R e = ea[r] * eb[c];
+    for (int j = 0; j < PAIRS * M; ++j) wc[q][j] = constAt<R>(w, (q * PAIRS * M + j) * RW);
 #pragma unroll
-      for (int t = 0; t < M; ++t) acc[t] = rfma(e, constAt<R>(w, ((r * NB + c) * M + t) * RW), acc[t]);
+  for (int q = 0; q < CHUNKS; ++q) {
+    if (q + AHEAD < CHUNKS) {
+#pragma unroll
+      for (int j = 0; j < PAIRS * M; ++j) wc[(q + AHEAD) % (AHEAD + 1)][j] = constAt<R>(w, ((q + AHEAD) * PAIRS * M + j) * RW);
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int k = 0; k < PAIRS; ++k) {
+      const int rc = q * PAIRS + k;
+      const R e = ea[rc / NB] * eb[rc % NB];
+#pragma unroll
+      for (int t = 0; t < M; ++t) acc[t] = rfma(e, wc[q % (AHEAD + 1)][k * M + t], acc[t]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
   }
   const R base = ma + mb;
 #pragma unroll
@@ -242,7 +260,7 @@ __device__ __forceinline__ code_ptr outerSumFixed(code_ptr ip, const Slots<R, fa
 
 template <typename R, bool LOG2, bool SPILL, int M>
 __device__ __forceinline__ code_ptr outerSumNB(code_ptr ip, int na, int nb, const Slots<R, SPILL>& S) {
-  if constexpr (!SPILL && M == 8) {
+  if constexpr (!SPILL && M == 8 && LOG2) {  // the unrolled form only where it pays: the float log2-domain kernel
     if (na == 8 && nb == 8) return outerSumFixed<R, LOG2, 8, 8, 8>(ip, S);
     if (na == 4 && nb == 4) return outerSumFixed<R, LOG2, 8, 4, 4>(ip, S);
   }
