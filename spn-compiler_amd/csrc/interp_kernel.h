@@ -14,13 +14,14 @@ struct InterpLaunch {
   void* out;                 // device: [n] of the compute type
   unsigned long long n;
   const void* tables;        // device: leaf-table pool of the compute type
-  void* spill;               // device: [numSpillSlots][gridDim.x * INTERP_BLOCK] of the compute type
+  void* spill;               // device: [gridDim.x][spillSlots][INTERP_BLOCK] of the compute type
   const uint32_t* staged;    // device: numStaged * 4 words (column, valueSlot, indexSlot, tableLen)
   uint32_t numStaged;
   uint32_t numFeatures;
   uint32_t featureType;      // spnc_hip::FeatureType as integer
   uint32_t featureMode;      // FEAT_STAGED / FEAT_DIRECT
   uint32_t ldsSlots;         // slots [0, ldsSlots) live in LDS, the rest in the spill tier
+  uint32_t spillSlots;       // number of slots in the spill tier
   uint32_t marginal;         // NaN features marginalise Gaussian leaves
 };
 

@@ -115,21 +115,43 @@ __device__ __forceinline__ uint32_t featureIndex(const void* __restrict__ in, ui
   }
 }
 
+// The first 64 words of an instruction, length word included, held in one vector register: lane j
+// holds word j, fetched with one coalesced load that the main loop issues for the next instruction
+// before it executes the current one. A word becomes a scalar through a lane read, which costs a few
+// cycles where a scalar load from the stream would cost a trip to the L2.
+struct Head {
+  static constexpr int WORDS = 64;
+  uint32_t lanes;
+  __device__ __forceinline__ uint32_t word(int j) const { return uint32_t(__builtin_amdgcn_readlane(int(lanes), j)); }
+};
+__device__ __forceinline__ Head loadHead(const uint32_t* codeGlobal, long at) {
+  Head h;
+  h.lanes = codeGlobal[at + (threadIdx.x & 63u)];
+  return h;
+}
+
 // SPILL = false: every slot of the program lives in LDS, reads and writes are branch-free, so
 // the compiler can batch the operand reads of an instruction.
 template <typename R, bool SPILL>
 struct Slots {
-  R* lds;                    // this lane's column: slot s at lds[s * B]
-  R* spill;                  // this lane's column: slot s at spill[(s - ldsSlots) * lanes]
-  unsigned long long lanes;
+  R* lds;        // this lane's column in LDS: slot s at lds[s * B]
+  R* spill;      // this lane's column in its block's part of the spill tier, moved back by ldsSlots slots:
+                 // slot s >= ldsSlots at spill[s * B], so both tiers use the same stride
   uint32_t ldsSlots;
+  // With a spill tier the base pointer is selected, not the access: one generic load or store
+  // per operand and no branch, so the operand accesses of an instruction can be in flight together.
+  __device__ __forceinline__ R* at(uint32_t s) const {
+    const unsigned long long inLds = (unsigned long long)(long long)(int32_t(s - ldsSlots) >> 31);  // all ones for LDS slots
+    const unsigned long long base = ((unsigned long long)lds & inLds) | ((unsigned long long)spill & ~inLds);
+    return reinterpret_cast<R*>(base) + s * B;
+  }
   __device__ __forceinline__ R rd(uint32_t s) const {
     if (!SPILL) return lds[s * B];
-    return s < ldsSlots ? lds[s * B] : spill[(unsigned long long)(s - ldsSlots) * lanes];
+    return *at(s);
   }
   __device__ __forceinline__ void wr(uint32_t s, R v) const {
-    if (!SPILL || s < ldsSlots) lds[s * B] = v;
-    else spill[(unsigned long long)(s - ldsSlots) * lanes] = v;
+    if (!SPILL) lds[s * B] = v;
+    else *at(s) = v;
   }
 };
 
@@ -198,20 +220,51 @@ __device__ __forceinline__ code_ptr outerSum(code_ptr ip, int na, const Slots<R,
   return w + long(na) * NB * M * RW;
 }
 
-// Fully unrolled form for operand vectors of a fixed, small size that all live in LDS: both
-// vectors are read into registers first, so that the multiply-accumulate part contains no LDS
-// access and its weights can stream in through wide scalar loads that overlap the arithmetic.
-template <typename R, bool LOG2, int M, int NA, int NB>
-__device__ __forceinline__ code_ptr outerSumFixed(code_ptr ip, const Slots<R, false>& S) {
-  typedef Math<R, LOG2> Mt;
-  constexpr int RW = sizeof(R) / 4;
-  code_ptr dsts = ip + 2, as = dsts + M, bs = as + NA, w = bs + NB;
-  R ea[NA], eb[NB];
-  R ma = R(-__builtin_huge_val()), mb = R(-__builtin_huge_val());
+// Outer sum of eight float sums on the matrix cores. One 4x4x1 instruction multiplies, in every
+// group of four lanes, four values of matrix A by four values of matrix B and accumulates the 16
+// products; with the A-broadcast controls (cbsz = 4, abid = b) all sixteen groups take A from
+// the four lanes of group b. So a vector register loaded with 64 consecutive weights (lane
+// 4*b + i holds the weight of sum i for product b) serves sixteen products, B is simply every
+// lane's own product exp(a_r - ma) * exp(b_c - mb), and accumulator register i of a lane ends up
+// with sum i of that lane's sample: no data crosses lanes outside the instruction itself.
+// The weights arrive through ordinary coalesced vector loads, requested before the operands.
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+template <int K, int KEND, int NB>
+struct MatrixSteps {
+  static __device__ __forceinline__ void run(const float* ea, const float* eb, const float (*A)[2], float4v& d0, float4v& d1) {
+    const float e = ea[K / NB] * eb[K % NB];
+    d0 = __builtin_amdgcn_mfma_f32_4x4x1f32(A[K / 16][0], e, d0, 4, K % 16, 0);
+    d1 = __builtin_amdgcn_mfma_f32_4x4x1f32(A[K / 16][1], e, d1, 4, K % 16, 0);
+    // Left alone, the scheduler forms all products first and holds them in registers, which costs occupancy.
+    if (K % 8 == 7) __builtin_amdgcn_sched_barrier(0);
+    MatrixSteps<K + 1, KEND, NB>::run(ea, eb, A, d0, d1);
+  }
+};
+template <int KEND, int NB>
+struct MatrixSteps<KEND, KEND, NB> {
+  static __device__ __forceinline__ void run(const float*, const float*, const float (*)[2], float4v&, float4v&) {}
+};
+
+template <bool LOG2, bool SPILL, int NA, int NB>
+__device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
+  typedef Math<float, LOG2> Mt;
+  constexpr int M = 8, K = NA * NB, GROUPS = K / 16;
+  constexpr int DST = 3, AS = DST + M, BS = AS + NA;  // positions in the head: length, opcode, M, then the slot lists
+  static_assert(BS + NB <= Head::WORDS, "the slot lists must lie within the prefetched head");
+  float A[GROUPS][2];
+  const float* wl = wGlobal + (threadIdx.x & 63u);
 #pragma unroll
-  for (int r = 0; r < NA; ++r) ea[r] = S.rd(as[r]);
+  for (int g = 0; g < GROUPS; ++g) {
+    A[g][0] = wl[g * 128];
+    A[g][1] = wl[g * 128 + 64];
+  }
+  float ea[NA], eb[NB];
+  float ma = -__builtin_huge_valf(), mb = -__builtin_huge_valf();
 #pragma unroll
-  for (int c = 0; c < NB; ++c) eb[c] = S.rd(bs[c]);
+  for (int r = 0; r < NA; ++r) ea[r] = S.rd(h.word(AS + r));
+#pragma unroll
+  for (int c = 0; c < NB; ++c) eb[c] = S.rd(h.word(BS + c));
 #pragma unroll
   for (int r = 0; r < NA; ++r) ma = rmax(ma, ea[r]);
 #pragma unroll
@@ -222,64 +275,93 @@ __device__ __forceinline__ code_ptr outerSumFixed(code_ptr ip, const Slots<R, fa
   for (int r = 0; r < NA; ++r) ea[r] = Mt::exp(ea[r] - ma);
 #pragma unroll
   for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(eb[c] - mb);
-  R acc[M];
+  float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+  MatrixSteps<0, K, NB>::run(ea, eb, A, d0, d1);
+  const float base = ma + mb;
 #pragma unroll
-  for (int t = 0; t < M; ++t) acc[t] = R(0);
-  // The weights arrive through scalar loads, whose wait counter is all-or-nothing: they are
-  // requested two chunks of PAIRS (r,c) pairs ahead and the scheduler is kept from moving the
-  // requests, so that two chunks of multiply-adds (and the other waves of the SIMD) cover the
-  // latency of a chunk's loads.
-  constexpr int PAIRS = (16 / RW) / M >= 1 ? (16 / RW) / M : 1, CHUNKS = NA * NB / PAIRS, AHEAD = 2;
-  static_assert(NA * NB % PAIRS == 0, "chunking must divide the weight matrix");
-  R wc[AHEAD + 1][PAIRS * M];
+  for (int t = 0; t < 4; ++t) S.wr(h.word(DST + t), base + Mt::log(d0[t]));
 #pragma unroll
-  for (int q = 0; q < AHEAD && q < CHUNKS; ++q)
-#pragma unroll
-    for (int j = 0; j < PAIRS * M; ++j) wc[q][j] = constAt<R>(w, (q * PAIRS * M + j) * RW);
-#pragma unroll
-  for (int q = 0; q < CHUNKS; ++q) {
-    if (q + AHEAD < CHUNKS) {
-#pragma unroll
-      for (int j = 0; j < PAIRS * M; ++j) wc[(q + AHEAD) % (AHEAD + 1)][j] = constAt<R>(w, ((q + AHEAD) * PAIRS * M + j) * RW);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int k = 0; k < PAIRS; ++k) {
-      const int rc = q * PAIRS + k;
-      const R e = ea[rc / NB] * eb[rc % NB];
-#pragma unroll
-      for (int t = 0; t < M; ++t) acc[t] = rfma(e, wc[q % (AHEAD + 1)][k * M + t], acc[t]);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  const R base = ma + mb;
-#pragma unroll
-  for (int t = 0; t < M; ++t) S.wr(dsts[t], base + Mt::log(acc[t]));
-  return w + NA * NB * M * RW;
+  for (int t = 0; t < 4; ++t) S.wr(h.word(DST + 4 + t), base + Mt::log(d1[t]));
+  return ip + 2 + M + NA + NB + K * M;
+}
+
+// The operand counts the program builder emits the matrix form for (matrixFormShape in interp_program.cpp).
+template <bool LOG2, bool SPILL>
+__device__ __forceinline__ code_ptr outerSumMatrixAny(code_ptr ip, const Head& h, int na, int nb, const float* wGlobal, const Slots<float, SPILL>& S) {
+  if (na == 8 && nb == 8) return outerSumMatrix<LOG2, SPILL, 8, 8>(ip, h, wGlobal, S);
+  if (na == 4 && nb == 4) return outerSumMatrix<LOG2, SPILL, 4, 4>(ip, h, wGlobal, S);
+  if (na == 4 && nb == 8) return outerSumMatrix<LOG2, SPILL, 4, 8>(ip, h, wGlobal, S);
+  if (na == 8 && nb == 4) return outerSumMatrix<LOG2, SPILL, 8, 4>(ip, h, wGlobal, S);
+  if (na == 2 && nb == 8) return outerSumMatrix<LOG2, SPILL, 2, 8>(ip, h, wGlobal, S);
+  return outerSumMatrix<LOG2, SPILL, 8, 2>(ip, h, wGlobal, S);
 }
 
 template <typename R, bool LOG2, bool SPILL, int M>
 __device__ __forceinline__ code_ptr outerSumNB(code_ptr ip, int na, int nb, const Slots<R, SPILL>& S) {
-  if constexpr (!SPILL && M == 8 && LOG2) {  // the unrolled form only where it pays: the float log2-domain kernel
-    if (na == 8 && nb == 8) return outerSumFixed<R, LOG2, 8, 8, 8>(ip, S);
-    if (na == 4 && nb == 4) return outerSumFixed<R, LOG2, 8, 4, 4>(ip, S);
-  }
   if (nb == 8) return outerSum<R, LOG2, SPILL, M, 8>(ip, na, S);
   if (nb == 4) return outerSum<R, LOG2, SPILL, M, 4>(ip, na, S);
   if (nb == 16) return outerSum<R, LOG2, SPILL, M, 16>(ip, na, S);
   return outerSum<R, LOG2, SPILL, M, 2>(ip, na, S);
 }
 
+// n products of G Gaussian leaves each. The records are independent, so they are taken four at
+// a time: all constants of a group arrive in a few wide scalar loads and all feature reads of a
+// group are in flight together, instead of one dependent load chain per product.
+template <typename R, bool SPILL, int G, bool stagedMode>
+__device__ __forceinline__ code_ptr prodBatch(code_ptr ip, int n, const Slots<R, SPILL>& S, const InterpLaunch& a, unsigned long long row) {
+  constexpr int RW = sizeof(R) / 4, LEAF = 1 + 3 * RW, REC = 1 + G * LEAF, P = 4;
+  ip += 2;
+  int done = 0;
+  for (; done + P <= n; done += P, ip += P * REC) {
+    R x[P][G];
+#pragma unroll
+    for (int q = 0; q < P; ++q)
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const uint32_t fw = ip[q * REC + 1 + j * LEAF];
+        x[q][j] = stagedMode ? S.rd(fw) : featureValue<R>(a.in, a.featureType, row + fw);
+      }
+#pragma unroll
+    for (int q = 0; q < P; ++q) {
+      R acc = R(0);
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const long at = q * REC + 1 + j * LEAF + 1;
+        const R d = x[q][j] - constAt<R>(ip, at);
+        R v = constAt<R>(ip, at + RW) + (d * d) * constAt<R>(ip, at + 2 * RW);
+        if (a.marginal) v = (x[q][j] != x[q][j]) ? R(0) : v;
+        acc += v;
+      }
+      S.wr(ip[q * REC], acc);
+    }
+  }
+  for (; done < n; ++done, ip += REC) {
+    R acc = R(0);
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+      const uint32_t fw = ip[1 + j * LEAF];
+      const R xv = stagedMode ? S.rd(fw) : featureValue<R>(a.in, a.featureType, row + fw);
+      const R d = xv - constAt<R>(ip, 2 + j * LEAF);
+      R v = constAt<R>(ip, 2 + j * LEAF + RW) + (d * d) * constAt<R>(ip, 2 + j * LEAF + 2 * RW);
+      if (a.marginal) v = (xv != xv) ? R(0) : v;
+      acc += v;
+    }
+    S.wr(ip[0], acc);
+  }
+  return ip;
+}
+
 // Executes one instruction other than OP_END and returns the pointer to the next one.
 template <typename R, bool LOG2, bool SPILL>
-__device__ __forceinline__ code_ptr execute(code_ptr ip, uint32_t w0, const Slots<R, SPILL>& S, const InterpLaunch& a,
-                                            const R* __restrict__ tables, unsigned long long row, bool stagedMode) {
+__device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Slots<R, SPILL>& S, const InterpLaunch& a,
+                                            const R* __restrict__ tables, unsigned long long row, bool stagedMode, code_ptr code0,
+                                            const uint32_t* codeGlobal) {
   typedef Math<R, LOG2> Mt;
   constexpr int RW = sizeof(R) / 4;
-  const uint32_t op = w0 & 0x7fu;
+  const uint32_t w0 = h.word(1), op = w0 & 0x7fu;
   if (op == OP_PROD) {
-    const uint32_t dst = ip[1];
-    const int ns = int(ip[2]), ng = int(ip[3]), nt = int(ip[4]);
+    const uint32_t dst = h.word(2);
+    const int ns = int(h.word(3)), ng = int(h.word(4)), nt = int(h.word(5));
     ip += 5;
     R acc = R(0);
 #pragma unroll 4
@@ -305,9 +387,24 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, uint32_t w0, const Slot
     S.wr(dst, acc);
     return ip;
   }
+  if (op == OP_PRODBATCH) {
+    const int n = int(w0 >> 8);
+    const uint32_t leaves = h.word(2);
+    // Staged features make the whole batch straight-line code; the direct form decides the input type per read.
+    if (stagedMode) {
+      if (leaves == 2) return prodBatch<R, SPILL, 2, true>(ip, n, S, a, row);
+      if (leaves == 1) return prodBatch<R, SPILL, 1, true>(ip, n, S, a, row);
+      if (leaves == 4) return prodBatch<R, SPILL, 4, true>(ip, n, S, a, row);
+      return prodBatch<R, SPILL, 3, true>(ip, n, S, a, row);
+    }
+    if (leaves == 2) return prodBatch<R, SPILL, 2, false>(ip, n, S, a, row);
+    if (leaves == 1) return prodBatch<R, SPILL, 1, false>(ip, n, S, a, row);
+    if (leaves == 4) return prodBatch<R, SPILL, 4, false>(ip, n, S, a, row);
+    return prodBatch<R, SPILL, 3, false>(ip, n, S, a, row);
+  }
   if (op == OP_SUM) {
     const int k = int(w0 >> 8);
-    const uint32_t dst = ip[1];
+    const uint32_t dst = h.word(2);
     ip += 2;
     if (k == 1) {
       S.wr(dst, S.rd(ip[0]) + constAt<R>(ip, 1));
@@ -325,14 +422,21 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, uint32_t w0, const Slot
   }
   if (op == OP_SUMLAYER) {
     const int k = int(w0 >> 8);
-    const uint32_t m = ip[1];
+    const uint32_t m = h.word(2);
     if (m == 8) return sumLayer<R, LOG2, SPILL, 8>(ip, k, S);
     if (m == 4) return sumLayer<R, LOG2, SPILL, 4>(ip, k, S);
     return sumLayer<R, LOG2, SPILL, 2>(ip, k, S);
   }
-  // OP_OUTERSUM
   const int na = int((w0 >> 8) & 0xffu), nb = int(w0 >> 16);
-  const uint32_t m = ip[1];
+  if constexpr (sizeof(R) == 4) {
+    if (op == OP_OUTERMM) {
+      // The weights start after the two header words, eight destinations and na + nb operands.
+      const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 10 + na + nb);
+      return outerSumMatrixAny<LOG2, SPILL>(ip, h, na, nb, wGlobal, S);
+    }
+  }
+  // OP_OUTERSUM
+  const uint32_t m = h.word(2);
   if (m == 8) return outerSumNB<R, LOG2, SPILL, 8>(ip, na, nb, S);
   if (m == 4) return outerSumNB<R, LOG2, SPILL, 4>(ip, na, nb, S);
   return outerSumNB<R, LOG2, SPILL, 2>(ip, na, nb, S);
@@ -351,18 +455,17 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
   R* __restrict__ out = static_cast<R*>(a.out);
   Slots<R, true> Sg;
   Sg.lds = reinterpret_cast<R*>(ldsRaw) + threadIdx.x;
-  Sg.lanes = (unsigned long long)gridDim.x * B;
-  Sg.spill = static_cast<R*>(a.spill) + (unsigned long long)blockIdx.x * B + threadIdx.x;
+  const unsigned long long lanes = (unsigned long long)gridDim.x * B;
+  Sg.spill = static_cast<R*>(a.spill) + (long long)blockIdx.x * a.spillSlots * B - (long long)a.ldsSlots * B + threadIdx.x;
   Sg.ldsSlots = a.ldsSlots;
   Slots<R, false> Sl;
   Sl.lds = Sg.lds;
-  Sl.lanes = Sg.lanes;
   Sl.spill = Sg.spill;
   Sl.ldsSlots = Sg.ldsSlots;
   const unsigned long long F = a.numFeatures;
   const bool stagedMode = a.featureMode == FEAT_STAGED;
 
-  for (unsigned long long base = (unsigned long long)blockIdx.x * B; base < a.n; base += Sg.lanes) {
+  for (unsigned long long base = (unsigned long long)blockIdx.x * B; base < a.n; base += lanes) {
     const unsigned long long i = base + threadIdx.x;
     const bool valid = i < a.n;
     const unsigned long long row = (valid ? i : a.n - 1) * F;  // idle lanes recompute the last sample
@@ -380,18 +483,49 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
       }
     }
 
-    code_ptr ip = code;
+    code_ptr ip = code;  // at the length word of the first instruction
+    Head h = loadHead(codeGlobal, 0);
     R result;
+#ifdef SPN_INTERP_PROFILE
+    // Diagnostic build: cycles the first wave of the grid spends per instruction class on its third tile.
+    long long cyc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    long long t0 = clock64();
+#endif
     for (;;) {
-      const uint32_t w0 = ip[0];
+      const uint32_t w0 = h.word(1);
       const bool spillPath = MODE == 2 || (MODE == 1 && (w0 & 0x80u));
       if ((w0 & 0x7fu) == OP_END) {
-        result = spillPath ? Sg.rd(ip[1]) : Sl.rd(ip[1]);
+        result = spillPath ? Sg.rd(h.word(2)) : Sl.rd(h.word(2));
         break;
       }
-      if (MODE != 0 && spillPath) ip = execute<R, LOG2, true>(ip, w0, Sg, a, tables, row, stagedMode);
-      else ip = execute<R, LOG2, false>(ip, w0, Sl, a, tables, row, stagedMode);
+      code_ptr next = ip + 1 + h.word(0);
+      const Head hn = loadHead(codeGlobal, next - code);  // in flight while this instruction executes
+      if (MODE != 0 && spillPath) execute<R, LOG2, true>(ip + 1, h, Sg, a, tables, row, stagedMode, code, codeGlobal);
+      else execute<R, LOG2, false>(ip + 1, h, Sl, a, tables, row, stagedMode, code, codeGlobal);
+      ip = next;
+      h = hn;
+#ifdef SPN_INTERP_PROFILE
+      {
+        const long long t1 = clock64();
+        const uint32_t op = w0 & 0x7fu;
+        int c = (op == OP_PROD || op == OP_PRODBATCH) ? 0 : (op == OP_OUTERSUM || op == OP_OUTERMM) ? (((w0 >> 16) == 8 ? 1 : 2) + (spillPath ? 2 : 0)) : 5;
+        if ((op == OP_PROD || op == OP_PRODBATCH) && spillPath) c = 6;
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+          if (q == c) {
+            cyc[q] += t1 - t0;
+            cnt[q]++;
+          }
+        t0 = t1;
+      }
+#endif
     }
+#ifdef SPN_INTERP_PROFILE
+    if (blockIdx.x == 0 && threadIdx.x == 0 && base == 2 * lanes)
+      printf("profile: prod %d/%lld outer8 %d/%lld outer4 %d/%lld outer8-spill %d/%lld outer4-spill %d/%lld other %d/%lld prod-spill %d/%lld\n",
+             cnt[0], cyc[0], cnt[1], cyc[1], cnt[2], cyc[2], cnt[3], cyc[3], cnt[4], cyc[4], cnt[5], cyc[5], cnt[6], cyc[6]);
+#endif
     if (valid) out[i] = Mt::finish(result);
   }
 }

@@ -23,6 +23,13 @@ struct Builder {
   Builder(const Graph& graph, InterpProgram& prog) : g(graph), p(prog) { scale = p.log2Domain ? 1.4426950408889634074 : 1.0; }
 
   void word(uint32_t w) { p.code.push_back(w); }
+  // Every instruction is preceded by one word holding its length, so that the kernel knows where
+  // the next instruction starts before it has decoded this one.
+  size_t begin() {
+    p.code.push_back(0);
+    return p.code.size() - 1;
+  }
+  void end(size_t at) { p.code[at] = uint32_t(p.code.size() - at - 1); }
   void real(double v) {
     if (p.f64) {
       uint64_t b;
@@ -43,6 +50,12 @@ struct Builder {
 
 namespace {
 InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t longRange, bool stagedLong);
+
+// Operand counts for which the kernel has a matrix-core outer sum (outerSumMatrixAny in interp_kernel.hip).
+bool matrixFormShape(uint32_t na, uint32_t nb) {
+  return (na == 8 && nb == 8) || (na == 4 && nb == 4) || (na == 4 && nb == 8) || (na == 8 && nb == 4) || (na == 2 && nb == 8) ||
+         (na == 8 && nb == 2);
+}
 }
 
 // Values that stay live for more than `longRange` instructions are numbered after all the others
@@ -52,27 +65,33 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
 // short pool fits the LDS share that lets four blocks reside on a CU, or failing that two.
 InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
   const bool f64 = o.computeType == ComputeType::F64;
-  const uint32_t fourBlocks = f64 ? 20 : 40, twoBlocks = f64 ? 36 : 72;
+  const uint32_t fourBlocks = o.interpShortSlots > 0 ? uint32_t(o.interpShortSlots) : (f64 ? 20 : 40), twoBlocks = f64 ? 36 : 72;
+  // Candidates differ in which values count as long-lived (and so may leave LDS) and in the tier of
+  // the staged features. Preferred: a short pool that lets four blocks share a CU, then one that
+  // lets two; among those the candidate that touches the spill tier least.
   InterpProgram best;
   bool have = false;
+  auto rank = [&](const InterpProgram& p) { return p.shortSlots <= fourBlocks ? 0 : (p.shortSlots <= twoBlocks ? 1 : 2); };
   auto better = [&](const InterpProgram& p) {
     if (!have) return true;
-    const bool p4 = p.shortSlots <= fourBlocks, b4 = best.shortSlots <= fourBlocks;
-    const bool p2 = p.shortSlots <= twoBlocks, b2 = best.shortSlots <= twoBlocks;
-    if (p4 != b4) return p4;
-    if (p4) return false;  // the earlier candidate keeps more values in LDS
-    if (p2 != b2) return p2;
-    if (p2) return false;
-    return p.shortSlots < best.shortSlots;
+    const int rp = rank(p), rb = rank(best);
+    if (rp != rb) return rp < rb;
+    if (rp == 2) return p.shortSlots < best.shortSlots;
+    return p.spillAccesses < best.spillAccesses;
   };
   for (bool stagedLong : {false, true}) {
-    for (uint32_t range : {0xffffffffu, 256u, 64u, 32u, 16u, 8u}) {
+    if (o.interpStagedLong >= 0 && stagedLong != (o.interpStagedLong == 1)) continue;
+    for (uint32_t range : {0xffffffffu, 256u, 128u, 64u, 32u, 16u, 8u}) {
+      if (o.interpLongRange >= 0) {
+        if (range != 0xffffffffu) break;  // a fixed range: one candidate per tier choice
+        range = uint32_t(o.interpLongRange);
+      }
       InterpProgram p = buildWithRange(g, o, range, stagedLong);
       if (better(p)) {
         best = std::move(p);
         have = true;
       }
-      if (best.shortSlots <= fourBlocks) return best;
+      if (best.spillAccesses == 0 && rank(best) == 0) return best;
     }
   }
   return best;
@@ -300,6 +319,46 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
     }
   };
 
+  auto emitProd = [&](uint32_t node, uint32_t dst, const std::vector<uint32_t>& srcs, const std::vector<uint32_t>& gs,
+                      const std::vector<uint32_t>& ts, uint32_t longFlag) {
+    const size_t at = b.begin();
+    b.word(OP_PROD | longFlag);
+    slotWord(dst);
+    b.word(uint32_t(srcs.size()));
+    b.word(uint32_t(gs.size()));
+    b.word(uint32_t(ts.size()));
+    for (uint32_t s : srcs) slotWord(slotOf[s]);
+    for (uint32_t c : gs) emitInlineLeaf(c);
+    for (uint32_t c : ts) emitInlineLeaf(c);
+    b.end(at);
+    b.txt << "  " << slotName(dst) << " = prod(" << srcs.size() << " slots, " << gs.size() << " gaussians, " << ts.size() << " tables)   ; node "
+          << node << "\n";
+  };
+  struct BatchEntry {
+    uint32_t node, dst;
+    std::vector<uint32_t> leaves;
+  };
+  std::vector<BatchEntry> batch;
+  uint32_t batchFlag = 0;
+  auto flushBatch = [&]() {
+    if (batch.empty()) return;
+    if (batch.size() == 1) {
+      emitProd(batch[0].node, batch[0].dst, {}, batch[0].leaves, {}, batchFlag);
+    } else {
+      const size_t at = b.begin();
+      b.word(OP_PRODBATCH | batchFlag | (uint32_t(batch.size()) << 8));
+      b.word(uint32_t(batch[0].leaves.size()));
+      for (const auto& e : batch) {
+        slotWord(e.dst);
+        for (uint32_t c : e.leaves) emitInlineLeaf(c);
+      }
+      b.end(at);
+      b.txt << "  " << slotName(batch[0].dst) << ".. = prodbatch(" << batch.size() << " products x " << batch[0].leaves.size()
+            << " gaussians)   ; nodes " << batch[0].node << "..\n";
+    }
+    batch.clear();
+  };
+
   for (uint32_t k = 0; k < instrs.size(); ++k) {
     const Instr& in = instrs[k];
     // Sources dying here release their slots before the destinations are chosen: every
@@ -317,6 +376,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
     for (uint32_t d : in.defs) longFlag |= (slotOf[d] & LONG_BIT) ? 0x80u : 0u;
     for (uint32_t sidx : in.srcs) longFlag |= (slotOf[sidx] & LONG_BIT) ? 0x80u : 0u;
     const auto& n = g.nodes[in.node];
+    if (in.op != OP_PROD) flushBatch();
     switch (in.op) {
       case OP_PROD: {
         std::vector<uint32_t> gs, ts;
@@ -327,20 +387,22 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
             if (inlined[c]) (isTable(c) ? ts : gs).push_back(c);
         }
         if (stagedLong && p.featureMode == FEAT_STAGED && !(gs.empty() && ts.empty())) longFlag |= 0x80u;
-        b.word(OP_PROD | longFlag);
-        slotWord(slotOf[in.node]);
-        b.word(uint32_t(in.srcs.size()));
-        b.word(uint32_t(gs.size()));
-        b.word(uint32_t(ts.size()));
-        for (uint32_t s : in.srcs) slotWord(slotOf[s]);
-        for (uint32_t c : gs) emitInlineLeaf(c);
-        for (uint32_t c : ts) emitInlineLeaf(c);
-        b.txt << "  " << slotName(slotOf[in.node]) << " = prod(" << in.srcs.size() << " slots, " << gs.size() << " gaussians, " << ts.size()
-              << " tables)   ; node " << in.node << "\n";
+        // Products of Gaussian leaves only, all of one size, that follow each other become one
+        // batch instruction: their records do not depend on each other, so the kernel works on
+        // several at a time.
+        if (in.srcs.empty() && ts.empty() && !gs.empty() && gs.size() <= 4) {
+          if (!batch.empty() && (batch.front().leaves.size() != gs.size() || batchFlag != longFlag)) flushBatch();
+          batchFlag = longFlag;
+          batch.push_back(BatchEntry{in.node, slotOf[in.node], gs});
+          break;
+        }
+        flushBatch();
+        emitProd(in.node, slotOf[in.node], in.srcs, gs, ts, longFlag);
         break;
       }
       case OP_SUM: {
         uint32_t cnt = uint32_t(n.children.size());
+        const size_t at = b.begin();
         b.word(OP_SUM | longFlag | (cnt << 8));
         slotWord(slotOf[in.node]);
         for (uint32_t j = 0; j < cnt; ++j) {
@@ -348,35 +410,47 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
           if (cnt == 1) b.real(b.logConst(n.weights[j]));  // single child: value + log weight
           else b.real(n.weights[j]);
         }
+        b.end(at);
         b.txt << "  " << slotName(slotOf[in.node]) << " = sum(" << cnt << " terms)   ; node " << in.node << "\n";
         break;
       }
       case OP_SUMLAYER: {
         uint32_t cnt = uint32_t(n.children.size());
         uint32_t m = uint32_t(in.defs.size());
+        const size_t at = b.begin();
         b.word(OP_SUMLAYER | longFlag | (cnt << 8));
         b.word(m);
         for (uint32_t d : in.defs) slotWord(slotOf[d]);
         for (uint32_t j = 0; j < cnt; ++j) slotWord(slotOf[n.children[j]]);
         for (uint32_t j = 0; j < cnt; ++j)
           for (uint32_t d : in.defs) b.real(g.nodes[d].weights[j]);
+        b.end(at);
         b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = sumlayer(" << m << " sums x " << cnt << " terms)   ; nodes " << in.defs[0] << "..\n";
         break;
       }
       case OP_OUTERSUM: {
-        const Outer& o = outerOf.at(n.children);
-        const uint32_t na = uint32_t(o.a.size()), nb = uint32_t(o.b.size());
+        const Outer& outer = outerOf.at(n.children);
+        const uint32_t na = uint32_t(outer.a.size()), nb = uint32_t(outer.b.size());
         uint32_t m = uint32_t(in.defs.size());
         // A single leftover sum is encoded as a layer of two identical sums writing the same slot.
         std::vector<uint32_t> defs = in.defs;
         if (m == 1) defs.push_back(in.defs[0]);
-        b.word(OP_OUTERSUM | longFlag | (na << 8) | (nb << 16));
+        const bool matrixForm = !p.f64 && defs.size() == 8 && o.interpMatrixCore && matrixFormShape(na, nb);
+        const size_t at = b.begin();
+        b.word((matrixForm ? OP_OUTERMM : OP_OUTERSUM) | longFlag | (na << 8) | (nb << 16));
         b.word(uint32_t(defs.size()));
         for (uint32_t d : defs) slotWord(slotOf[d]);
-        for (uint32_t a : o.a) slotWord(slotOf[a]);
-        for (uint32_t c : o.b) slotWord(slotOf[c]);
-        for (uint32_t j = 0; j < na * nb; ++j)
-          for (uint32_t d : defs) b.real(g.nodes[d].weights[j]);
+        for (uint32_t a : outer.a) slotWord(slotOf[a]);
+        for (uint32_t c : outer.b) slotWord(slotOf[c]);
+        if (matrixForm) {
+          for (uint32_t grp = 0; grp < na * nb / 16; ++grp)
+            for (uint32_t half = 0; half < 2; ++half)
+              for (uint32_t lane = 0; lane < 64; ++lane) b.real(g.nodes[defs[half * 4 + lane % 4]].weights[grp * 16 + lane / 4]);
+        } else {
+          for (uint32_t j = 0; j < na * nb; ++j)
+            for (uint32_t d : defs) b.real(g.nodes[d].weights[j]);
+        }
+        b.end(at);
         b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = outersum(" << m << " sums x " << na << "x" << nb << " products)   ; nodes " << in.defs[0]
               << "..\n";
         break;
@@ -388,8 +462,13 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
     for (uint32_t d : in.defs)
       if (d != g.root() && lastUse[d] <= k) releaseSlot(slotOf[d]);
   }
-  b.word(OP_END | ((slotOf[g.root()] & LONG_BIT) ? 0x80u : 0u));
-  slotWord(slotOf[g.root()]);
+  flushBatch();
+  {
+    const size_t at = b.begin();
+    b.word(OP_END | ((slotOf[g.root()] & LONG_BIT) ? 0x80u : 0u));
+    slotWord(slotOf[g.root()]);
+    b.end(at);
+  }
   for (size_t pos : longWords) p.code[pos] = highWater + (p.code[pos] & ~LONG_BIT);
   for (auto& sf : p.staged) {
     if (sf.valueSlot != NONE && (sf.valueSlot & LONG_BIT)) sf.valueSlot = highWater + (sf.valueSlot & ~LONG_BIT);
@@ -398,6 +477,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   p.shortSlots = highWater;
   p.numSlots = highWater + longCount;
   p.numInstructions = uint32_t(instrs.size());
+  p.spillAccesses = uint32_t(longWords.size());
   std::ostringstream hdr;
   hdr << "; interpreter program for SPN '" << g.name << "': " << instrs.size() << " instructions, " << p.code.size() << " words, "
       << p.numSlots << " value slots (" << p.reservedSlots << " staged features, " << (p.numSlots - p.shortSlots) << " long-lived), compute " << (p.f64 ? "f64" : "f32")

@@ -13,6 +13,8 @@
 
 namespace spnc_hip {
 
+// The stream is a sequence of [length][instruction words...]: the length word counts the words of
+// the instruction that follows it.
 // Opcodes (low 7 bits of an instruction's first word; bit 7 is set when the instruction reads or
 // writes a long-lived slot; the upper 24 bits hold counts).
 enum InterpOp : uint32_t {
@@ -22,6 +24,12 @@ enum InterpOp : uint32_t {
   OP_SUMLAYER = 3,  // [op|k<<8][M][dst*M] k*slot, k*M weights        M sums over the same k children (M in 2,4,8)
   OP_OUTERSUM = 4,  // [op|NA<<8|NB<<16][M][dst*M] NA*slot, NB*slot, NA*NB*M weights
                     //   M sums over all products a_r * b_c of two operand vectors, products never materialised
+  OP_OUTERMM = 6,   // [op|NA<<8|NB<<16][8][dst*8] NA*slot, NB*slot, NA*NB*8 weights in matrix-core order
+                    //   OUTERSUM for float, eight sums and NA*NB a multiple of 16: weight of product k = r*NB + c and
+                    //   sum t sits at word (k/16)*128 + (t/4)*64 + (k%16)*4 + t%4, i.e. 64-word rows that one
+                    //   wavefront loads with one coalesced access and that feed sixteen 4x4x1 matrix instructions
+  OP_PRODBATCH = 5, // [op|n<<8][G] n*(dst, G*(feat, mean, coef, den))
+                    //   n products of G Gaussian leaves each; the records are independent of each other
 };
 
 // How leaves obtain their feature value.
@@ -49,6 +57,7 @@ struct InterpProgram {
   uint32_t shortSlots = 0;    // slots [0, shortSlots) are the busy ones; [shortSlots, numSlots) hold long-lived values
   uint32_t reservedSlots = 0; // leading slots pinned to staged features
   uint32_t numInstructions = 0;
+  uint32_t spillAccesses = 0; // slot words naming a long-lived slot: reads and writes of the spill tier per sample when only the short pool is in LDS
   std::string listing;        // human-readable form, for "dump-ir"
 };
 

@@ -349,7 +349,9 @@ void Kernel::ensureDevice() {
     int nb = 0;
     hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, interpMode_, ldsBytes_, &nb), "occupancy query");
     blocksPerCU_ = std::max(1, nb);
-    hipCheck(hipMalloc(&dCode_, prog_.code.size() * 4), "hipMalloc(program)");
+    // The kernel touches the cache lines that follow an instruction's weights, so the stream is padded past its end.
+    hipCheck(hipMalloc(&dCode_, prog_.code.size() * 4 + 512), "hipMalloc(program)");
+    hipCheck(hipMemset(dCode_, 0, prog_.code.size() * 4 + 512), "program padding");
     hipCheck(hipMemcpy(dCode_, prog_.code.data(), prog_.code.size() * 4, hipMemcpyHostToDevice), "program upload");
     if (!prog_.tables.empty()) {
       hipCheck(hipMalloc(&dTables_, prog_.tables.size() * rb), "hipMalloc(tables)");
@@ -436,6 +438,7 @@ void Kernel::launch(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
     a.featureType = featureType_;
     a.featureMode = prog_.featureMode;
     a.ldsSlots = ldsSlots_;
+    a.spillSlots = prog_.numSlots - ldsSlots_;
     a.marginal = marginal_ ? 1u : 0u;
     hipCheck(launchInterpreter(a, prog_.f64, prog_.log2Domain, interpMode_, grid, ldsBytes_, stream), "interpreter launch");
   }

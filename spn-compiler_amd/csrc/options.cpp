@@ -79,6 +79,8 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       else throw std::runtime_error("Could not parse option value " + val + " for " + key);
     } else if (key == "hip-log2-domain") {
       o.log2Domain = parseBool(val);
+    } else if (key == "hip-interp-matrix-core") {
+      o.interpMatrixCore = parseBool(val);
     } else if (key == "hip-samples-per-lane") {
       o.samplesPerLane = parseInt(key, val);
       if (o.samplesPerLane < 0 || o.samplesPerLane > 16) throw std::runtime_error("hip-samples-per-lane must be in [0,16]");
@@ -90,6 +92,17 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       o.eagerIndices = parseBool(val);
     } else if (key == "hip-joint-tables") {
       o.jointTables = parseBool(val);
+    } else if (key == "hip-interp-short-slots") {
+      o.interpShortSlots = parseInt(key, val);
+      if (o.interpShortSlots < 0 || o.interpShortSlots > 160) throw std::runtime_error("hip-interp-short-slots must be in [0,160]");
+    } else if (key == "hip-interp-staged-features") {
+      if (val == "lds") o.interpStagedLong = 0;
+      else if (val == "spill") o.interpStagedLong = 1;
+      else if (val == "auto") o.interpStagedLong = -1;
+      else throw std::runtime_error("hip-interp-staged-features must be lds, spill or auto");
+    } else if (key == "hip-interp-long-range") {
+      o.interpLongRange = parseInt(key, val);
+      if (o.interpLongRange < -1) throw std::runtime_error("hip-interp-long-range must be -1 or a count of instructions");
     } else if (key == "hip-min-blocks-per-cu") {
       o.minBlocksPerCU = parseInt(key, val);
       if (o.minBlocksPerCU < 0 || o.minBlocksPerCU > 8) throw std::runtime_error("hip-min-blocks-per-cu must be in [0,8]");

@@ -347,6 +347,45 @@ Graph buildGraph(const RawQuery& q) {
       }
     }
   }
+  // Sums over a complete outer product of two operand vectors: M sums share the ordered child list
+  // [prod(a_0,b_0), ..., prod(a_NA-1,b_NB-1)] and nothing else reads those products. Since
+  // exp(a_r + b_c - ma - mb) = exp(a_r - ma) * exp(b_c - mb), the group costs NA + NB exponentials, not M*NA*NB.
+  // Where that factored form is cheaper than the per-sum accounting above, it is the algorithmic minimum.
+  std::map<std::vector<uint32_t>, uint64_t> groups;
+  for (const auto& n : g.nodes)
+    if (n.kind == NodeKind::Sum && n.children.size() >= 4) groups[n.children]++;
+  for (const auto& entry : groups) {
+    const std::vector<uint32_t>& kids = entry.first;
+    const uint64_t members = entry.second, k = kids.size();
+    bool ok = true;
+    for (uint32_t c : kids) {
+      const auto& pn = g.nodes[c];
+      if (pn.kind != NodeKind::Product || pn.children.size() != 2 || pn.uses != members) ok = false;
+    }
+    if (!ok) continue;
+    uint64_t nb = 1;
+    while (nb < k && g.nodes[kids[nb]].children[0] == g.nodes[kids[0]].children[0]) ++nb;
+    if (nb < 2 || k % nb != 0 || k / nb < 2) continue;
+    const uint64_t na = k / nb;
+    for (uint64_t r = 0; r < na && ok; ++r)
+      for (uint64_t c = 0; c < nb && ok; ++c) {
+        const auto& pn = g.nodes[kids[r * nb + c]];
+        ok = pn.children[0] == g.nodes[kids[r * nb]].children[0] && pn.children[1] == g.nodes[kids[c]].children[1];
+      }
+    std::vector<uint32_t> sorted = kids;
+    std::sort(sorted.begin(), sorted.end());
+    if (std::adjacent_find(sorted.begin(), sorted.end()) != sorted.end()) ok = false;
+    if (!ok) continue;
+    // Per-sum accounting of the group, products included (k >= 4, so the n-ary form was the one charged).
+    const uint64_t naiveFlops = members * 5 * k + k, naiveTrans = members * (k + 1);
+    // Factored: two maxima and shifts (2 per operand), NA*NB products of exponentials, M*NA*NB multiply-adds,
+    // a logarithm and two adds per sum.
+    const uint64_t factFlops = 2 * (na + nb) + k + members * k + 2 * members, factTrans = na + nb + members;
+    if (factFlops + 3 * factTrans < naiveFlops + 3 * naiveTrans) {
+      st.flopsMin = st.flopsMin - naiveFlops + factFlops;
+      st.transMin = st.transMin - naiveTrans + factTrans;
+    }
+  }
   return g;
 }
 

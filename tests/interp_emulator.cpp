@@ -56,8 +56,11 @@ int main(int argc, char** argv) {
         if (s.valueSlot != UINT32_MAX) slot.at(s.valueSlot) = float(x[s.column]);
         if (s.indexSlot != UINT32_MAX) slot.at(s.indexSlot) = float(index(x[s.column], s.tableLen));
       }
-      size_t pc = 0;
+      size_t pc = 0, expectedEnd = 0;
       for (;;) {
+        if (pc != expectedEnd) throw std::runtime_error("length word disagrees with the instruction before word " + std::to_string(pc));
+        expectedEnd = pc + 1 + c.at(pc);
+        ++pc;
         const uint32_t w0 = c.at(pc), op = w0 & 0x7f;
         const bool flagged = w0 & 0x80;
         auto rd = [&](uint32_t s) {
@@ -91,6 +94,23 @@ int main(int argc, char** argv) {
           }
           wr(dst, acc);
           pc = q;
+        } else if (op == OP_PRODBATCH) {
+          const uint32_t n = w0 >> 8, G = c.at(pc + 1);
+          if (n < 2 || G < 1 || G > 4) throw std::runtime_error("malformed product batch at word " + std::to_string(pc));
+          size_t q = pc + 2;
+          for (uint32_t i = 0; i < n; ++i) {
+            const uint32_t dst = c.at(q++);
+            float acc = 0;
+            for (uint32_t j = 0; j < G; ++j, q += 4) {
+              const float xv = p.featureMode == FEAT_STAGED ? rd(c.at(q)) : float(x[c.at(q)]);
+              const float d = xv - asFloat(c.at(q + 1));
+              float v = asFloat(c.at(q + 2)) + d * d * asFloat(c.at(q + 3));
+              if (g.supportMarginal && xv != xv) v = 0;
+              acc += v;
+            }
+            wr(dst, acc);
+          }
+          pc = q;
         } else if (op == OP_SUM) {
           const uint32_t k = w0 >> 8, dst = c.at(pc + 1);
           size_t q = pc + 2;
@@ -116,8 +136,13 @@ int main(int argc, char** argv) {
             for (uint32_t j = 0; j < k; ++j) res[t] += ex(rd(c.at(k0 + j)) - m) * asFloat(c.at(w + j * M + t));
           for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), m + lg(res[t]));
           pc = w + size_t(k) * M;
-        } else if (op == OP_OUTERSUM) {
+        } else if (op == OP_OUTERSUM || op == OP_OUTERMM) {
           const uint32_t na = (w0 >> 8) & 0xff, nb = w0 >> 16, M = c.at(pc + 1);
+          if (op == OP_OUTERMM && (M != 8 || (na * nb) % 16 != 0)) throw std::runtime_error("malformed matrix-form outer sum at word " + std::to_string(pc));
+          // Matrix form: product k and sum t at (k/16)*128 + (t/4)*64 + (k%16)*4 + t%4.
+          auto weightAt = [&](size_t w, uint32_t k, uint32_t t) {
+            return asFloat(op == OP_OUTERMM ? c.at(w + (k / 16) * 128 + (t / 4) * 64 + (k % 16) * 4 + t % 4) : c.at(w + size_t(k) * M + t));
+          };
           const size_t d0 = pc + 2, a0 = d0 + M, b0 = a0 + na, w = b0 + nb;
           float ma = -INFINITY, mb = -INFINITY;
           for (uint32_t r = 0; r < na; ++r) ma = std::fmax(ma, rd(c.at(a0 + r)));
@@ -128,7 +153,7 @@ int main(int argc, char** argv) {
           for (uint32_t t = 0; t < M; ++t)
             for (uint32_t r = 0; r < na; ++r)
               for (uint32_t cc = 0; cc < nb; ++cc)
-                res[t] += ex(rd(c.at(a0 + r)) - ma) * ex(rd(c.at(b0 + cc)) - mb) * asFloat(c.at(w + (size_t(r) * nb + cc) * M + t));
+                res[t] += ex(rd(c.at(a0 + r)) - ma) * ex(rd(c.at(b0 + cc)) - mb) * weightAt(w, r * nb + cc, t);
           for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), ma + mb + lg(res[t]));
           pc = w + size_t(na) * nb * M;
         } else {
