@@ -23,6 +23,17 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X FP32 vector, published
 FP64_VECTOR_PEAK_TFLOPS = 78.6   # MI355X FP64 vector, published
 
+# HBM bytes per launch from the counter runs summarised in profiles/<kernel>_<workload>.txt:
+# workload -> (samples per launch, bytes). Only valid for that launch size and the default options.
+MEASURED_HBM_TRAFFIC = {
+    "c1": (67108864, 1879038771),
+    "c2": (16777216, 1142188819),
+    "c3": (8388608, 3495427481),
+    "c4": (4194304, 8368113601),
+    "c5": (16777216, 1141495178),
+    "c5_f64": (16777216, 1212272946),
+}
+
 
 def make_inputs(name, cfg, n, torch, device):
     """Synthetic inputs of the configuration's shape and distribution, generated on the device."""
@@ -48,6 +59,7 @@ def make_inputs(name, cfg, n, torch, device):
 def measure(name, n, steps, warmup, torch, device, extra_options=None):
     from spnc import synthetic as syn
     from spnc.hip import HIPCompiler
+    workload_key, extra_given = name, bool(extra_options)
     if name == "c5_f64":   # configuration 5 computed in float64 log-space
         name, extra_options = "c5", dict(extra_options or {}, **{"hip-compute-type": "float64"})
     cfg = syn.CONFIGS[name]
@@ -123,14 +135,10 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None):
     }
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by what a
     # plain copy of known size reads on the same counters); recorded per workload under profiles/.
-    try:
-        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            entry = json.load(f).get(name)
-        if entry and entry.get("samples") == n:
-            roof["traffic"] = entry["bytes_per_launch"]
-            roof["traffic_over_algorithmic"] = round(entry["bytes_per_launch"] / (bytes_per_sample * n), 3)
-    except (OSError, ValueError):
-        pass
+    entry = MEASURED_HBM_TRAFFIC.get(workload_key)
+    if entry and entry[0] == n and not extra_given:
+        roof["traffic"] = entry[1]
+        roof["traffic_over_algorithmic"] = round(entry[1] / (bytes_per_sample * n), 3)
     res = {
         "workload": name, "desc": cfg["desc"], "n": n, "samples_per_s": n * steps / wall, "ms_per_step": wall / steps * 1e3,
         "roofline": roof, "compile_s": round(compile_s, 2), "nodes": info["num_nodes"], "finite": finite,
