@@ -234,10 +234,17 @@ template <int K, int KEND, int NB>
 struct MatrixSteps {
   static __device__ __forceinline__ void run(const float* ea, const float* eb, const float (*A)[2], float4v& d0, float4v& d1) {
     const float e = ea[K / NB] * eb[K % NB];
-    d0 = __builtin_amdgcn_mfma_f32_4x4x1f32(A[K / 16][0], e, d0, 4, K % 16, 0);
-    d1 = __builtin_amdgcn_mfma_f32_4x4x1f32(A[K / 16][1], e, d1, 4, K % 16, 0);
-    // Left alone, the scheduler forms all products first and holds them in registers, which costs occupancy.
-    if (K % 8 == 7) __builtin_amdgcn_sched_barrier(0);
+    // One assembly statement per product keeps the two accumulator chains interleaved: left to the compiler they
+    // run one after the other, with every product held in a register in between (64 registers for an 8x8 region)
+    // and a stall between each pair of dependent instructions. An instruction that accumulates onto the result
+    // of the one before the previous needs two wait states in between (the other chain's instruction and the s_nop
+    // provide three), and the s_nop also separates the product's multiply from its first use.
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_mfma_f32_4x4x1_16b_f32 %0, %2, %4, %0 cbsz:4 abid:%5\n\t"
+        "v_mfma_f32_4x4x1_16b_f32 %1, %3, %4, %1 cbsz:4 abid:%5"
+        : "+v"(d0), "+v"(d1)
+        : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "n"(K % 16));
     MatrixSteps<K + 1, KEND, NB>::run(ea, eb, A, d0, d1);
   }
 };

@@ -65,18 +65,21 @@ bool matrixFormShape(uint32_t na, uint32_t nb) {
 // short pool fits the LDS share that lets four blocks reside on a CU, or failing that two.
 InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
   const bool f64 = o.computeType == ComputeType::F64;
-  const uint32_t fourBlocks = o.interpShortSlots > 0 ? uint32_t(o.interpShortSlots) : (f64 ? 20 : 40), twoBlocks = f64 ? 36 : 72;
+  // Short-pool sizes (slots of 256 values) that let six, four or two blocks share the 160 KiB of a CU.
+  const uint32_t sixBlocks = o.interpShortSlots > 0 ? uint32_t(o.interpShortSlots) : (f64 ? 13 : 26), fourBlocks = f64 ? 20 : 40,
+                 twoBlocks = f64 ? 36 : 72;
   // Candidates differ in which values count as long-lived (and so may leave LDS) and in the tier of
-  // the staged features. Preferred: a short pool that lets four blocks share a CU, then one that
-  // lets two; among those the candidate that touches the spill tier least.
+  // the staged features. Preferred: the most blocks per CU (measured on a RAT-SPN: 9.0 ms with six,
+  // 9.7 ms with four, 10.1 ms with eight blocks of 16 slots); among equals the candidate that
+  // touches the spill tier least.
   InterpProgram best;
   bool have = false;
-  auto rank = [&](const InterpProgram& p) { return p.shortSlots <= fourBlocks ? 0 : (p.shortSlots <= twoBlocks ? 1 : 2); };
+  auto rank = [&](const InterpProgram& p) { return p.shortSlots <= sixBlocks ? 0 : (p.shortSlots <= fourBlocks ? 1 : (p.shortSlots <= twoBlocks ? 2 : 3)); };
   auto better = [&](const InterpProgram& p) {
     if (!have) return true;
     const int rp = rank(p), rb = rank(best);
     if (rp != rb) return rp < rb;
-    if (rp == 2) return p.shortSlots < best.shortSlots;
+    if (rp == 3) return p.shortSlots < best.shortSlots;
     return p.spillAccesses < best.spillAccesses;
   };
   for (bool stagedLong : {false, true}) {
