@@ -137,7 +137,12 @@ struct Slots {
   R* lds;        // this lane's column in LDS: slot s at lds[s * B]
   R* spill;      // this lane's column in its block's part of the spill tier, moved back by ldsSlots slots:
                  // slot s >= ldsSlots at spill[s * B], so both tiers use the same stride
+  R* spillBlock; // the same without the lane: wave-uniform, so spill accesses can take a scalar base and the lane as offset
   uint32_t ldsSlots;
+  __device__ __forceinline__ R rdLds(uint32_t s) const { return lds[s * B]; }
+  __device__ __forceinline__ R rdSpill(uint32_t s) const { return spillBlock[(unsigned long long)s * B + threadIdx.x]; }
+  __device__ __forceinline__ void wrLds(uint32_t s, R v) const { lds[s * B] = v; }
+  __device__ __forceinline__ void wrSpill(uint32_t s, R v) const { spillBlock[(unsigned long long)s * B + threadIdx.x] = v; }
   // With a spill tier the base pointer is selected, not the access: one generic load or store
   // per operand and no branch, so the operand accesses of an instruction can be in flight together.
   __device__ __forceinline__ R* at(uint32_t s) const {
@@ -253,7 +258,7 @@ struct MatrixSteps<KEND, KEND, NB> {
   static __device__ __forceinline__ void run(const float*, const float*, const float (*)[2], float4v&, float4v&) {}
 };
 
-template <bool LOG2, bool SPILL, int NA, int NB>
+template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB>
 __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
   typedef Math<float, LOG2> Mt;
   constexpr int M = 8, K = NA * NB, GROUPS = K / 16;
@@ -268,10 +273,31 @@ __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, c
   }
   float ea[NA], eb[NB];
   float ma = -__builtin_huge_valf(), mb = -__builtin_huge_valf();
+  // Flagged instructions: the tier bits say per slot list where it lives (valid when exactly the short pool is
+  // in LDS), so a list is read with LDS instructions or with scalar-base global loads; mixed lists and other
+  // LDS splits take the select-the-base form.
+  const uint32_t tierA = TIERED ? (h.word(1) >> 24) & 3u : 2u, tierB = TIERED ? (h.word(1) >> 26) & 3u : 2u,
+                 tierD = TIERED ? (h.word(1) >> 28) & 3u : 2u;
+  if (!SPILL || tierA == 0) {
 #pragma unroll
-  for (int r = 0; r < NA; ++r) ea[r] = S.rd(h.word(AS + r));
+    for (int r = 0; r < NA; ++r) ea[r] = S.rdLds(h.word(AS + r));
+  } else if (tierA == 1) {
 #pragma unroll
-  for (int c = 0; c < NB; ++c) eb[c] = S.rd(h.word(BS + c));
+    for (int r = 0; r < NA; ++r) ea[r] = S.rdSpill(h.word(AS + r));
+  } else {
+#pragma unroll
+    for (int r = 0; r < NA; ++r) ea[r] = S.rd(h.word(AS + r));
+  }
+  if (!SPILL || tierB == 0) {
+#pragma unroll
+    for (int c = 0; c < NB; ++c) eb[c] = S.rdLds(h.word(BS + c));
+  } else if (tierB == 1) {
+#pragma unroll
+    for (int c = 0; c < NB; ++c) eb[c] = S.rdSpill(h.word(BS + c));
+  } else {
+#pragma unroll
+    for (int c = 0; c < NB; ++c) eb[c] = S.rd(h.word(BS + c));
+  }
 #pragma unroll
   for (int r = 0; r < NA; ++r) ma = rmax(ma, ea[r]);
 #pragma unroll
@@ -285,22 +311,34 @@ __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, c
   float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
   MatrixSteps<0, K, NB>::run(ea, eb, A, d0, d1);
   const float base = ma + mb;
+  float res[M];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) S.wr(h.word(DST + t), base + Mt::log(d0[t]));
+  for (int t = 0; t < 4; ++t) {
+    res[t] = base + Mt::log(d0[t]);
+    res[4 + t] = base + Mt::log(d1[t]);
+  }
+  if (!SPILL || tierD == 0) {
 #pragma unroll
-  for (int t = 0; t < 4; ++t) S.wr(h.word(DST + 4 + t), base + Mt::log(d1[t]));
+    for (int t = 0; t < M; ++t) S.wrLds(h.word(DST + t), res[t]);
+  } else if (tierD == 1) {
+#pragma unroll
+    for (int t = 0; t < M; ++t) S.wrSpill(h.word(DST + t), res[t]);
+  } else {
+#pragma unroll
+    for (int t = 0; t < M; ++t) S.wr(h.word(DST + t), res[t]);
+  }
   return ip + 2 + M + NA + NB + K * M;
 }
 
 // The operand counts the program builder emits the matrix form for (matrixFormShape in interp_program.cpp).
-template <bool LOG2, bool SPILL>
+template <bool LOG2, bool SPILL, bool TIERED>
 __device__ __forceinline__ code_ptr outerSumMatrixAny(code_ptr ip, const Head& h, int na, int nb, const float* wGlobal, const Slots<float, SPILL>& S) {
-  if (na == 8 && nb == 8) return outerSumMatrix<LOG2, SPILL, 8, 8>(ip, h, wGlobal, S);
-  if (na == 4 && nb == 4) return outerSumMatrix<LOG2, SPILL, 4, 4>(ip, h, wGlobal, S);
-  if (na == 4 && nb == 8) return outerSumMatrix<LOG2, SPILL, 4, 8>(ip, h, wGlobal, S);
-  if (na == 8 && nb == 4) return outerSumMatrix<LOG2, SPILL, 8, 4>(ip, h, wGlobal, S);
-  if (na == 2 && nb == 8) return outerSumMatrix<LOG2, SPILL, 2, 8>(ip, h, wGlobal, S);
-  return outerSumMatrix<LOG2, SPILL, 8, 2>(ip, h, wGlobal, S);
+  if (na == 8 && nb == 8) return outerSumMatrix<LOG2, SPILL, TIERED, 8, 8>(ip, h, wGlobal, S);
+  if (na == 4 && nb == 4) return outerSumMatrix<LOG2, SPILL, TIERED, 4, 4>(ip, h, wGlobal, S);
+  if (na == 4 && nb == 8) return outerSumMatrix<LOG2, SPILL, TIERED, 4, 8>(ip, h, wGlobal, S);
+  if (na == 8 && nb == 4) return outerSumMatrix<LOG2, SPILL, TIERED, 8, 4>(ip, h, wGlobal, S);
+  if (na == 2 && nb == 8) return outerSumMatrix<LOG2, SPILL, TIERED, 2, 8>(ip, h, wGlobal, S);
+  return outerSumMatrix<LOG2, SPILL, TIERED, 8, 2>(ip, h, wGlobal, S);
 }
 
 template <typename R, bool LOG2, bool SPILL, int M>
@@ -359,7 +397,7 @@ __device__ __forceinline__ code_ptr prodBatch(code_ptr ip, int n, const Slots<R,
 }
 
 // Executes one instruction other than OP_END and returns the pointer to the next one.
-template <typename R, bool LOG2, bool SPILL>
+template <typename R, bool LOG2, bool SPILL, bool TIERED>
 __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Slots<R, SPILL>& S, const InterpLaunch& a,
                                             const R* __restrict__ tables, unsigned long long row, bool stagedMode, code_ptr code0,
                                             const uint32_t* codeGlobal) {
@@ -434,12 +472,12 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
     if (m == 4) return sumLayer<R, LOG2, SPILL, 4>(ip, k, S);
     return sumLayer<R, LOG2, SPILL, 2>(ip, k, S);
   }
-  const int na = int((w0 >> 8) & 0xffu), nb = int(w0 >> 16);
+  const int na = int((w0 >> 8) & 0xffu), nb = int((w0 >> 16) & 0xffu);
   if constexpr (sizeof(R) == 4) {
     if (op == OP_OUTERMM) {
       // The weights start after the two header words, eight destinations and na + nb operands.
       const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 10 + na + nb);
-      return outerSumMatrixAny<LOG2, SPILL>(ip, h, na, nb, wGlobal, S);
+      return outerSumMatrixAny<LOG2, SPILL, TIERED>(ip, h, na, nb, wGlobal, S);
     }
   }
   // OP_OUTERSUM
@@ -463,11 +501,13 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
   Slots<R, true> Sg;
   Sg.lds = reinterpret_cast<R*>(ldsRaw) + threadIdx.x;
   const unsigned long long lanes = (unsigned long long)gridDim.x * B;
-  Sg.spill = static_cast<R*>(a.spill) + (long long)blockIdx.x * a.spillSlots * B - (long long)a.ldsSlots * B + threadIdx.x;
+  Sg.spillBlock = static_cast<R*>(a.spill) + (long long)blockIdx.x * a.spillSlots * B - (long long)a.ldsSlots * B;
+  Sg.spill = Sg.spillBlock + threadIdx.x;
   Sg.ldsSlots = a.ldsSlots;
   Slots<R, false> Sl;
   Sl.lds = Sg.lds;
   Sl.spill = Sg.spill;
+  Sl.spillBlock = Sg.spillBlock;
   Sl.ldsSlots = Sg.ldsSlots;
   const unsigned long long F = a.numFeatures;
   const bool stagedMode = a.featureMode == FEAT_STAGED;
@@ -508,15 +548,15 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
       }
       code_ptr next = ip + 1 + h.word(0);
       const Head hn = loadHead(codeGlobal, next - code);  // in flight while this instruction executes
-      if (MODE != 0 && spillPath) execute<R, LOG2, true>(ip + 1, h, Sg, a, tables, row, stagedMode, code, codeGlobal);
-      else execute<R, LOG2, false>(ip + 1, h, Sl, a, tables, row, stagedMode, code, codeGlobal);
+      if (MODE != 0 && spillPath) execute<R, LOG2, true, MODE == 1>(ip + 1, h, Sg, a, tables, row, stagedMode, code, codeGlobal);
+      else execute<R, LOG2, false, false>(ip + 1, h, Sl, a, tables, row, stagedMode, code, codeGlobal);
       ip = next;
       h = hn;
 #ifdef SPN_INTERP_PROFILE
       {
         const long long t1 = clock64();
         const uint32_t op = w0 & 0x7fu;
-        int c = (op == OP_PROD || op == OP_PRODBATCH) ? 0 : (op == OP_OUTERSUM || op == OP_OUTERMM) ? (((w0 >> 16) == 8 ? 1 : 2) + (spillPath ? 2 : 0)) : 5;
+        int c = (op == OP_PROD || op == OP_PRODBATCH) ? 0 : (op == OP_OUTERSUM || op == OP_OUTERMM) ? ((((w0 >> 16) & 0xffu) == 8 ? 1 : 2) + (spillPath ? 2 : 0)) : 5;
         if ((op == OP_PROD || op == OP_PRODBATCH) && spillPath) c = 6;
 #pragma unroll
         for (int q = 0; q < 8; ++q)

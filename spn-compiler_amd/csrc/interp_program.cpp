@@ -440,7 +440,15 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
         if (m == 1) defs.push_back(in.defs[0]);
         const bool matrixForm = !p.f64 && defs.size() == 8 && o.interpMatrixCore && matrixFormShape(na, nb);
         const size_t at = b.begin();
-        b.word((matrixForm ? OP_OUTERMM : OP_OUTERSUM) | longFlag | (na << 8) | (nb << 16));
+        // Matrix form: bits 24-29 say where each slot list lives (0 all in the short pool, 1 all in the long pool,
+        // 2 mixed), so the kernel picks the access instructions per list, not per slot.
+        auto tierOf = [&](const std::vector<uint32_t>& nodes) {
+          uint32_t longOnes = 0;
+          for (uint32_t x : nodes) longOnes += (slotOf[x] & LONG_BIT) ? 1 : 0;
+          return longOnes == 0 ? 0u : (longOnes == nodes.size() ? 1u : 2u);
+        };
+        const uint32_t tiers = matrixForm ? (tierOf(outer.a) << 24) | (tierOf(outer.b) << 26) | (tierOf(defs) << 28) : 0u;
+        b.word((matrixForm ? OP_OUTERMM : OP_OUTERSUM) | longFlag | (na << 8) | (nb << 16) | tiers);
         b.word(uint32_t(defs.size()));
         for (uint32_t d : defs) slotWord(slotOf[d]);
         for (uint32_t a : outer.a) slotWord(slotOf[a]);

@@ -24,7 +24,8 @@ enum InterpOp : uint32_t {
   OP_SUMLAYER = 3,  // [op|k<<8][M][dst*M] k*slot, k*M weights        M sums over the same k children (M in 2,4,8)
   OP_OUTERSUM = 4,  // [op|NA<<8|NB<<16][M][dst*M] NA*slot, NB*slot, NA*NB*M weights
                     //   M sums over all products a_r * b_c of two operand vectors, products never materialised
-  OP_OUTERMM = 6,   // [op|NA<<8|NB<<16][8][dst*8] NA*slot, NB*slot, NA*NB*8 weights in matrix-core order
+  OP_OUTERMM = 6,   // [op|NA<<8|NB<<16|tiers<<24][8][dst*8] NA*slot, NB*slot, NA*NB*8 weights in matrix-core order
+                    //   tiers: two bits each for the a, b and dst lists: 0 all short-pool slots, 1 all long-pool, 2 mixed
                     //   OUTERSUM for float, eight sums and NA*NB a multiple of 16: weight of product k = r*NB + c and
                     //   sum t sits at word (k/16)*128 + (t/4)*64 + (k%16)*4 + t%4, i.e. 64-word rows that one
                     //   wavefront loads with one coalesced access and that feed sixteen 4x4x1 matrix instructions

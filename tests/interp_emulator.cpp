@@ -137,7 +137,16 @@ int main(int argc, char** argv) {
           for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), m + lg(res[t]));
           pc = w + size_t(k) * M;
         } else if (op == OP_OUTERSUM || op == OP_OUTERMM) {
-          const uint32_t na = (w0 >> 8) & 0xff, nb = w0 >> 16, M = c.at(pc + 1);
+          const uint32_t na = (w0 >> 8) & 0xff, nb = (w0 >> 16) & 0xff, M = c.at(pc + 1);
+          if (op == OP_OUTERMM) {  // the tier bits must describe the slot lists
+            auto tier = [&](size_t first, uint32_t count) {
+              uint32_t longOnes = 0;
+              for (uint32_t j = 0; j < count; ++j) longOnes += c.at(first + j) >= p.shortSlots ? 1 : 0;
+              return longOnes == 0 ? 0u : (longOnes == count ? 1u : 2u);
+            };
+            const uint32_t want = (tier(pc + 2 + M, na) << 24) | (tier(pc + 2 + M + na, nb) << 26) | (tier(pc + 2, M) << 28);
+            if ((w0 & 0x3f000000u) != want) throw std::runtime_error("tier bits disagree with the slot lists at word " + std::to_string(pc));
+          }
           if (op == OP_OUTERMM && (M != 8 || (na * nb) % 16 != 0)) throw std::runtime_error("malformed matrix-form outer sum at word " + std::to_string(pc));
           // Matrix form: product k and sum t at (k/16)*128 + (t/4)*64 + (k%16)*4 + t%4.
           auto weightAt = [&](size_t w, uint32_t k, uint32_t t) {
