@@ -137,7 +137,7 @@ struct Emitter {
                        [&](uint32_t x, uint32_t y) { return rowLen(g.nodes[x].feature) < rowLen(g.nodes[y].feature); });
       for (size_t k = 0; k + 1 < leaves.size(); k += 2) {
         const size_t ra = rowLen(g.nodes[leaves[k]].feature), rb = rowLen(g.nodes[leaves[k + 1]].feature);
-        if (ra * rb <= 160) candidates.push_back({ra * rb - ra - rb, leaves[k], leaves[k + 1]});
+        if (ra * rb <= size_t(o.jointMaxEntries)) candidates.push_back({ra * rb - ra - rb, leaves[k], leaves[k + 1]});
       }
     }
     std::stable_sort(candidates.begin(), candidates.end(), [](const Candidate& x, const Candidate& y) { return x.extra < y.extra; });

@@ -352,7 +352,7 @@ __device__ __forceinline__ code_ptr outerSumNB(code_ptr ip, int na, int nb, cons
 // n products of G Gaussian leaves each. The records are independent, so they are taken four at
 // a time: all constants of a group arrive in a few wide scalar loads and all feature reads of a
 // group are in flight together, instead of one dependent load chain per product.
-template <typename R, bool SPILL, int G, bool stagedMode>
+template <typename R, bool SPILL, int G, bool stagedMode, bool MARGINAL>
 __device__ __forceinline__ code_ptr prodBatch(code_ptr ip, int n, const Slots<R, SPILL>& S, const InterpLaunch& a, unsigned long long row) {
   constexpr int RW = sizeof(R) / 4, LEAF = 1 + 3 * RW, REC = 1 + G * LEAF, P = 4;
   ip += 2;
@@ -373,8 +373,8 @@ __device__ __forceinline__ code_ptr prodBatch(code_ptr ip, int n, const Slots<R,
       for (int j = 0; j < G; ++j) {
         const long at = q * REC + 1 + j * LEAF + 1;
         const R d = x[q][j] - constAt<R>(ip, at);
-        R v = constAt<R>(ip, at + RW) + (d * d) * constAt<R>(ip, at + 2 * RW);
-        if (a.marginal) v = (x[q][j] != x[q][j]) ? R(0) : v;
+        R v = rfma(d, d, constAt<R>(ip, at + RW)) * constAt<R>(ip, at + 2 * RW);
+        if (MARGINAL && a.marginal) v = (x[q][j] != x[q][j]) ? R(0) : v;
         acc += v;
       }
       S.wr(ip[q * REC], acc);
@@ -387,8 +387,8 @@ __device__ __forceinline__ code_ptr prodBatch(code_ptr ip, int n, const Slots<R,
       const uint32_t fw = ip[1 + j * LEAF];
       const R xv = stagedMode ? S.rd(fw) : featureValue<R>(a.in, a.featureType, row + fw);
       const R d = xv - constAt<R>(ip, 2 + j * LEAF);
-      R v = constAt<R>(ip, 2 + j * LEAF + RW) + (d * d) * constAt<R>(ip, 2 + j * LEAF + 2 * RW);
-      if (a.marginal) v = (xv != xv) ? R(0) : v;
+      R v = rfma(d, d, constAt<R>(ip, 2 + j * LEAF + RW)) * constAt<R>(ip, 2 + j * LEAF + 2 * RW);
+      if (MARGINAL && a.marginal) v = (xv != xv) ? R(0) : v;
       acc += v;
     }
     S.wr(ip[0], acc);
@@ -415,11 +415,11 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
 #pragma unroll 2
     for (int j = 0; j < ng; ++j) {
       const uint32_t fw = ip[0];
-      const R mean = constAt<R>(ip, 1), coef = constAt<R>(ip, 1 + RW), den = constAt<R>(ip, 1 + 2 * RW);
+      const R mean = constAt<R>(ip, 1), shift = constAt<R>(ip, 1 + RW), den = constAt<R>(ip, 1 + 2 * RW);
       ip += 1 + 3 * RW;
       const R x = stagedMode ? S.rd(fw) : featureValue<R>(a.in, a.featureType, row + fw);
       const R d = x - mean;
-      R v = coef + (d * d) * den;
+      R v = rfma(d, d, shift) * den;
       if (a.marginal) v = (x != x) ? R(0) : v;
       acc += v;
     }
@@ -436,16 +436,23 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
     const int n = int(w0 >> 8);
     const uint32_t leaves = h.word(2);
     // Staged features make the whole batch straight-line code; the direct form decides the input type per read.
-    if (stagedMode) {
-      if (leaves == 2) return prodBatch<R, SPILL, 2, true>(ip, n, S, a, row);
-      if (leaves == 1) return prodBatch<R, SPILL, 1, true>(ip, n, S, a, row);
-      if (leaves == 4) return prodBatch<R, SPILL, 4, true>(ip, n, S, a, row);
-      return prodBatch<R, SPILL, 3, true>(ip, n, S, a, row);
+    // Without marginal support (the common staged case) the NaN select is not compiled in at all.
+    if (stagedMode && !a.marginal) {
+      if (leaves == 2) return prodBatch<R, SPILL, 2, true, false>(ip, n, S, a, row);
+      if (leaves == 1) return prodBatch<R, SPILL, 1, true, false>(ip, n, S, a, row);
+      if (leaves == 4) return prodBatch<R, SPILL, 4, true, false>(ip, n, S, a, row);
+      return prodBatch<R, SPILL, 3, true, false>(ip, n, S, a, row);
     }
-    if (leaves == 2) return prodBatch<R, SPILL, 2, false>(ip, n, S, a, row);
-    if (leaves == 1) return prodBatch<R, SPILL, 1, false>(ip, n, S, a, row);
-    if (leaves == 4) return prodBatch<R, SPILL, 4, false>(ip, n, S, a, row);
-    return prodBatch<R, SPILL, 3, false>(ip, n, S, a, row);
+    if (stagedMode) {
+      if (leaves == 2) return prodBatch<R, SPILL, 2, true, true>(ip, n, S, a, row);
+      if (leaves == 1) return prodBatch<R, SPILL, 1, true, true>(ip, n, S, a, row);
+      if (leaves == 4) return prodBatch<R, SPILL, 4, true, true>(ip, n, S, a, row);
+      return prodBatch<R, SPILL, 3, true, true>(ip, n, S, a, row);
+    }
+    if (leaves == 2) return prodBatch<R, SPILL, 2, false, true>(ip, n, S, a, row);
+    if (leaves == 1) return prodBatch<R, SPILL, 1, false, true>(ip, n, S, a, row);
+    if (leaves == 4) return prodBatch<R, SPILL, 4, false, true>(ip, n, S, a, row);
+    return prodBatch<R, SPILL, 3, false, true>(ip, n, S, a, row);
   }
   if (op == OP_SUM) {
     const int k = int(w0 >> 8);

@@ -312,7 +312,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       if (p.featureMode == FEAT_STAGED) slotWord(valueSlotOf[leaf.feature]);
       else b.word(leaf.feature);
       b.real(leaf.mean);
-      b.real(coef * b.scale);
+      b.real(coef / den);  // value = den * (d * d + coef / den): one multiply-add and one multiply, each with one constant
       b.real(den * b.scale);
     } else {
       if (p.featureMode == FEAT_STAGED) slotWord(indexSlotOf[leaf.feature]);

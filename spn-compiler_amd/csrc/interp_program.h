@@ -19,7 +19,8 @@ namespace spnc_hip {
 // writes a long-lived slot; the upper 24 bits hold counts).
 enum InterpOp : uint32_t {
   OP_END = 0,       // [op][src]                       result = slot src
-  OP_PROD = 1,      // [op][dst][ns][ng][nt] ns*slot, ng*(feat, mean, coef, den), nt*(feat, tableOffset, tableLen)
+  OP_PROD = 1,      // [op][dst][ns][ng][nt] ns*slot, ng*(feat, mean, shift, den), nt*(feat, tableOffset, tableLen)
+                    //   Gaussian leaf value = den * ((x - mean)^2 + shift), den = -1/(2 sigma^2) in the kernel's log unit
   OP_SUM = 2,       // [op|k<<8][dst] k*(slot, weight)                 one weighted sum
   OP_SUMLAYER = 3,  // [op|k<<8][M][dst*M] k*slot, k*M weights        M sums over the same k children (M in 2,4,8)
   OP_OUTERSUM = 4,  // [op|NA<<8|NB<<16][M][dst*M] NA*slot, NB*slot, NA*NB*M weights
@@ -29,7 +30,7 @@ enum InterpOp : uint32_t {
                     //   OUTERSUM for float, eight sums and NA*NB a multiple of 16: weight of product k = r*NB + c and
                     //   sum t sits at word (k/16)*128 + (t/4)*64 + (k%16)*4 + t%4, i.e. 64-word rows that one
                     //   wavefront loads with one coalesced access and that feed sixteen 4x4x1 matrix instructions
-  OP_PRODBATCH = 5, // [op|n<<8][G] n*(dst, G*(feat, mean, coef, den))
+  OP_PRODBATCH = 5, // [op|n<<8][G] n*(dst, G*(feat, mean, shift, den))
                     //   n products of G Gaussian leaves each; the records are independent of each other
 };
 

@@ -103,6 +103,9 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
     } else if (key == "hip-interp-long-range") {
       o.interpLongRange = parseInt(key, val);
       if (o.interpLongRange < -1) throw std::runtime_error("hip-interp-long-range must be -1 or a count of instructions");
+    } else if (key == "hip-joint-max-entries") {
+      o.jointMaxEntries = parseInt(key, val);
+      if (o.jointMaxEntries < 0 || o.jointMaxEntries > 4096) throw std::runtime_error("hip-joint-max-entries must be in [0,4096]");
     } else if (key == "hip-min-blocks-per-cu") {
       o.minBlocksPerCU = parseInt(key, val);
       if (o.minBlocksPerCU < 0 || o.minBlocksPerCU > 8) throw std::runtime_error("hip-min-blocks-per-cu must be in [0,8]");

@@ -34,6 +34,7 @@ struct CompileOptions {
   bool nontemporalLoads = true;                // "hip-nontemporal-loads": mark input loads as streaming
   bool eagerIndices = true;                    // "hip-eager-indices": compute table indices of all features first
   bool jointTables = true;                     // "hip-joint-tables": pair table leaves of a product into joint tables
+  int jointMaxEntries = 160;                   // "hip-joint-max-entries": largest joint table (entries) a pair of table leaves may get
   int interpShortSlots = 0;                    // "hip-interp-short-slots": LDS value slots per lane the interpreter program aims for (0 = automatic)
   bool interpMatrixCore = true;                // "hip-interp-matrix-core": float outer sums of eight sums run on the matrix cores
   int interpStagedLong = -1;                   // "hip-interp-staged-features": lds|spill (-1 = automatic): tier of the staged input features

@@ -84,7 +84,7 @@ int main(int argc, char** argv) {
           for (uint32_t j = 0; j < ng; ++j, q += 4) {
             const float xv = p.featureMode == FEAT_STAGED ? rd(c.at(q)) : float(x[c.at(q)]);
             const float d = xv - asFloat(c.at(q + 1));
-            float v = asFloat(c.at(q + 2)) + d * d * asFloat(c.at(q + 3));
+            float v = (d * d + asFloat(c.at(q + 2))) * asFloat(c.at(q + 3));
             if (g.supportMarginal && xv != xv) v = 0;
             acc += v;
           }
@@ -104,7 +104,7 @@ int main(int argc, char** argv) {
             for (uint32_t j = 0; j < G; ++j, q += 4) {
               const float xv = p.featureMode == FEAT_STAGED ? rd(c.at(q)) : float(x[c.at(q)]);
               const float d = xv - asFloat(c.at(q + 1));
-              float v = asFloat(c.at(q + 2)) + d * d * asFloat(c.at(q + 3));
+              float v = (d * d + asFloat(c.at(q + 2))) * asFloat(c.at(q + 3));
               if (g.supportMarginal && xv != xv) v = 0;
               acc += v;
             }
