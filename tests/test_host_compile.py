@@ -99,6 +99,10 @@ def test_option_handling(native):
     os.remove(k.fileName())
     with pytest.raises(RuntimeError, match="Could not parse option value"):
         compile_query(native, path, **{"hip-kernel": "magic"})
+    with pytest.raises(RuntimeError, match="hip-interp-staged-features must be lds, spill or auto"):
+        compile_query(native, path, **{"hip-kernel": "interpreter", "hip-interp-staged-features": "hbm"})
+    with pytest.raises(RuntimeError, match="hip-joint-max-entries must be in"):
+        compile_query(native, path, **{"hip-joint-max-entries": -3})
 
 
 def test_graph_stats_file(native, tmp_path):
@@ -186,7 +190,17 @@ def test_generated_source_variants(native):
     assert k.info()["kernel_kind"] == 2 and "sumlayer" not in k.source() and "sum(4 terms)" in k.source()
     os.remove(k.fileName())
     k = compile_spn(native, syn.c4_spn(), "float32")
-    assert k.info()["kernel_kind"] == 2 and "outersum(8 sums x 8x8 products)" in k.source()
+    src = k.source()
+    assert k.info()["kernel_kind"] == 2 and "outersum(8 sums x 8x8 products)" in src
+    # leaf products come in batches of eight (two leaf regions of four), 80 leaf regions pairs in all
+    assert src.count("prodbatch(8 products x 2 gaussians)") == 80 and " = prod(" not in src
+    # outer-product sums are priced in their factored form: far fewer exponentials than sum terms
+    i = k.info()
+    assert i["trans_min"] < i["sum_terms"] // 10 and i["flops_min"] < 2 * i["sum_terms"]
+    os.remove(k.fileName())
+    # the program builder honours the tier and pool-size options
+    k = compile_spn(native, syn.c4_spn(), "float32", **{"hip-interp-staged-features": "lds", "hip-interp-long-range": 8, "hip-interp-short-slots": 40})
+    assert "136 value slots (32 staged features, 96 long-lived)" in k.source()
     os.remove(k.fileName())
 
 
