@@ -117,7 +117,7 @@ struct Emitter {
     // the pair of indices, J[i][j] = T_a[i] (+ or *) T_b[j], combined in double. One LDS read and one
     // integer multiply-add then stand in for two LDS reads and one add; LDS reads are what bounds
     // table-heavy SPNs. Pairing stops when the pool would outgrow its LDS budget.
-    const size_t realBytes = f64 ? 8 : 4, budget = 62 * 1024;  // LDS instruction offsets reach 64 KiB
+    const size_t realBytes = f64 ? 8 : 4, budget = size_t(o.tableBudgetKiB) * 1024;  // at most 62 KiB: LDS instruction offsets reach 64 KiB
     size_t plain = 0;
     for (uint32_t i = 0; i < g.nodes.size(); ++i)
       if (isTable(i)) plain += rowLen(g.nodes[i].feature);

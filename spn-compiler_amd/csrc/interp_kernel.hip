@@ -235,27 +235,49 @@ __device__ __forceinline__ code_ptr outerSum(code_ptr ip, int na, const Slots<R,
 // The weights arrive through ordinary coalesced vector loads, requested before the operands.
 typedef float float4v __attribute__((ext_vector_type(4)));
 
+// Step K of the chain: both accumulators take product e_K, and the multiply that forms e_(K+2)
+// sits between the two matrix instructions. One assembly statement per step keeps the two
+// accumulator chains interleaved: left to the compiler they run one after the other, with every
+// product held in a register in between (64 registers for an 8x8 region) and a stall between each
+// pair of dependent instructions. Spacing rules, measured on gfx950 with a known-answer kernel:
+// a matrix instruction that reads a register which a vector instruction has just written needs
+// wait states in between and the hardware does not provide them (wrong results with none, and now
+// and then with only another matrix instruction in between), hence products are formed two
+// steps ahead and the first statement opens with s_nop; a matrix instruction may follow the one
+// it accumulates onto after one independent matrix instruction; vector instructions that read a
+// matrix result are held back by the hardware.
 template <int K, int KEND, int NB>
 struct MatrixSteps {
-  static __device__ __forceinline__ void run(const float* ea, const float* eb, const float (*A)[2], float4v& d0, float4v& d1) {
-    const float e = ea[K / NB] * eb[K % NB];
-    // One assembly statement per product keeps the two accumulator chains interleaved: left to the compiler they
-    // run one after the other, with every product held in a register in between (64 registers for an 8x8 region)
-    // and a stall between each pair of dependent instructions. An instruction that accumulates onto the result
-    // of the one before the previous needs two wait states in between (the other chain's instruction and the s_nop
-    // provide three), and the s_nop also separates the product's multiply from its first use.
-    asm volatile(
-        "s_nop 1\n\t"
-        "v_mfma_f32_4x4x1_16b_f32 %0, %2, %4, %0 cbsz:4 abid:%5\n\t"
-        "v_mfma_f32_4x4x1_16b_f32 %1, %3, %4, %1 cbsz:4 abid:%5"
-        : "+v"(d0), "+v"(d1)
-        : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "n"(K % 16));
-    MatrixSteps<K + 1, KEND, NB>::run(ea, eb, A, d0, d1);
+  static __device__ __forceinline__ void run(const float* ea, const float* eb, const float (*A)[2], float4v& d0, float4v& d1, float e,
+                                             float e1) {
+    if constexpr (K + 2 < KEND) {
+      float e2;
+      if constexpr (K == 0) {
+        asm volatile(
+            "s_nop 1\n\t"
+            "v_mfma_f32_4x4x1_16b_f32 %0, %3, %5, %0 cbsz:4 abid:%8\n\t"
+            "v_mul_f32 %2, %6, %7\n\t"
+            "v_mfma_f32_4x4x1_16b_f32 %1, %4, %5, %1 cbsz:4 abid:%8"
+            : "+v"(d0), "+v"(d1), "=&v"(e2)
+            : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "v"(ea[(K + 2) / NB]), "v"(eb[(K + 2) % NB]), "n"(K % 16), "v"(e1));
+      } else {
+        asm volatile(
+            "v_mfma_f32_4x4x1_16b_f32 %0, %3, %5, %0 cbsz:4 abid:%8\n\t"
+            "v_mul_f32 %2, %6, %7\n\t"
+            "v_mfma_f32_4x4x1_16b_f32 %1, %4, %5, %1 cbsz:4 abid:%8"
+            : "+v"(d0), "+v"(d1), "=&v"(e2)
+            : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "v"(ea[(K + 2) / NB]), "v"(eb[(K + 2) % NB]), "n"(K % 16), "v"(e1));
+      }
+      MatrixSteps<K + 1, KEND, NB>::run(ea, eb, A, d0, d1, e1, e2);
+    } else {
+      asm volatile(
+          "v_mfma_f32_4x4x1_16b_f32 %0, %2, %4, %0 cbsz:4 abid:%5\n\t"
+          "v_mfma_f32_4x4x1_16b_f32 %1, %3, %4, %1 cbsz:4 abid:%5"
+          : "+v"(d0), "+v"(d1)
+          : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "n"(K % 16), "v"(e1));
+      if constexpr (K + 1 < KEND) MatrixSteps<K + 1, KEND, NB>::run(ea, eb, A, d0, d1, e1, e1);
+    }
   }
-};
-template <int KEND, int NB>
-struct MatrixSteps<KEND, KEND, NB> {
-  static __device__ __forceinline__ void run(const float*, const float*, const float (*)[2], float4v&, float4v&) {}
 };
 
 template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB>
@@ -309,7 +331,7 @@ __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, c
 #pragma unroll
   for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(eb[c] - mb);
   float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
-  MatrixSteps<0, K, NB>::run(ea, eb, A, d0, d1);
+  MatrixSteps<0, K, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
   const float base = ma + mb;
   float res[M];
 #pragma unroll

@@ -489,6 +489,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   p.numSlots = highWater + longCount;
   p.numInstructions = uint32_t(instrs.size());
   p.spillAccesses = uint32_t(longWords.size());
+  p.ldsSlotLimit = uint32_t(o.interpLdsSlots);
   std::ostringstream hdr;
   hdr << "; interpreter program for SPN '" << g.name << "': " << instrs.size() << " instructions, " << p.code.size() << " words, "
       << p.numSlots << " value slots (" << p.reservedSlots << " staged features, " << (p.numSlots - p.shortSlots) << " long-lived), compute " << (p.f64 ? "f64" : "f32")

@@ -49,7 +49,7 @@ std::vector<char> compileWithHipRtc(const JitSource& js, int optLevel) {
 }
 
 // ---- kernel file: magic, then tagged little-endian fields ----
-const char kMagic[8] = {'S', 'P', 'N', 'C', 'H', 'I', 'P', 1};
+const char kMagic[8] = {'S', 'P', 'N', 'C', 'H', 'I', 'P', 2};
 
 struct Writer {
   std::vector<char> buf;
@@ -217,6 +217,7 @@ void Kernel::save(const std::string& path) const {
     w.u32(prog_.shortSlots);
     w.u32(prog_.reservedSlots);
     w.u32(prog_.numInstructions);
+    w.u32(prog_.ldsSlotLimit);
   }
   FILE* f = std::fopen(path.c_str(), "wb");
   if (!f) fatal("COMPILATION ERROR: cannot write kernel file " + path);
@@ -272,6 +273,7 @@ std::unique_ptr<Kernel> Kernel::load(const std::string& kernelFile) {
     k->prog_.shortSlots = r.u32();
     k->prog_.reservedSlots = r.u32();
     k->prog_.numInstructions = r.u32();
+    k->prog_.ldsSlotLimit = r.u32();
     k->inputAlign_ = k->bytesPerFeature_;
   } else {
     fatal("RUNTIME ERROR: unknown kernel kind in " + kernelFile);
@@ -335,6 +337,7 @@ void Kernel::ensureDevice() {
     hipCheck(interpreterMaxLds(prog_.f64, prog_.log2Domain, &maxBlock), "LDS limit query");
     size_t budget = std::min<size_t>(maxBlock, size_t(ldsPerCU) / 2);
     uint32_t cap = uint32_t(budget / (INTERP_BLOCK * rb));
+    if (prog_.ldsSlotLimit) cap = std::min(cap, prog_.ldsSlotLimit);
     if (prog_.numSlots <= cap) {
       ldsSlots_ = prog_.numSlots;
       interpMode_ = 0;

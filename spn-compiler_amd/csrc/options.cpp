@@ -95,6 +95,9 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
     } else if (key == "hip-interp-short-slots") {
       o.interpShortSlots = parseInt(key, val);
       if (o.interpShortSlots < 0 || o.interpShortSlots > 160) throw std::runtime_error("hip-interp-short-slots must be in [0,160]");
+    } else if (key == "hip-interp-lds-slots") {
+      o.interpLdsSlots = parseInt(key, val);
+      if (o.interpLdsSlots < 0 || o.interpLdsSlots > 160) throw std::runtime_error("hip-interp-lds-slots must be in [0,160]");
     } else if (key == "hip-interp-staged-features") {
       if (val == "lds") o.interpStagedLong = 0;
       else if (val == "spill") o.interpStagedLong = 1;
@@ -103,6 +106,9 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
     } else if (key == "hip-interp-long-range") {
       o.interpLongRange = parseInt(key, val);
       if (o.interpLongRange < -1) throw std::runtime_error("hip-interp-long-range must be -1 or a count of instructions");
+    } else if (key == "hip-table-budget-kib") {
+      o.tableBudgetKiB = parseInt(key, val);
+      if (o.tableBudgetKiB < 0 || o.tableBudgetKiB > 62) throw std::runtime_error("hip-table-budget-kib must be in [0,62]");
     } else if (key == "hip-joint-max-entries") {
       o.jointMaxEntries = parseInt(key, val);
       if (o.jointMaxEntries < 0 || o.jointMaxEntries > 4096) throw std::runtime_error("hip-joint-max-entries must be in [0,4096]");

@@ -34,9 +34,11 @@ struct CompileOptions {
   bool nontemporalLoads = true;                // "hip-nontemporal-loads": mark input loads as streaming
   bool eagerIndices = true;                    // "hip-eager-indices": compute table indices of all features first
   bool jointTables = true;                     // "hip-joint-tables": pair table leaves of a product into joint tables
+  int tableBudgetKiB = 62;                     // "hip-table-budget-kib": LDS the table pool may grow to when leaves are paired into joint tables
   int jointMaxEntries = 160;                   // "hip-joint-max-entries": largest joint table (entries) a pair of table leaves may get
   int interpShortSlots = 0;                    // "hip-interp-short-slots": LDS value slots per lane the interpreter program aims for (0 = automatic)
   bool interpMatrixCore = true;                // "hip-interp-matrix-core": float outer sums of eight sums run on the matrix cores
+  int interpLdsSlots = 0;                      // "hip-interp-lds-slots": upper bound on the value slots the launcher keeps in LDS (0 = automatic)
   int interpStagedLong = -1;                   // "hip-interp-staged-features": lds|spill (-1 = automatic): tier of the staged input features
   long interpLongRange = -1;                   // "hip-interp-long-range": values living longer than this many instructions go to the long-lived pool (-1 = automatic)
   int minBlocksPerCU = 0;                      // "hip-min-blocks-per-cu": register budget hint for the generated kernel (0 = none)

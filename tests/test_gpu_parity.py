@@ -386,3 +386,64 @@ def test_random_spns(native, seed):
         if not has_gauss:
             got = run(compile_spn(native, spn, "int32", **{}), Xi)
             check_f32(got, oracle_model(spn, "int32"), Xi.astype(np.uint32), False)
+
+
+def _region_graph(seed, shapes, num_features=12, marginal=False):
+    """Region graph whose sum groups cover given (left, right) operand counts: `shapes` lists, from
+    the root region down, how many nodes the left child region holds; the right child is the rest of
+    the chain and always holds eight sums (the last one: `shapes[-1][1]` leaf products)."""
+    from spnc.structure import Gaussian, Product, Sum
+    rng = np.random.default_rng(seed)
+
+    def leaves(scope, count):
+        return [Product(children=[Gaussian(mean=float(rng.normal()), stdev=float(rng.uniform(0.3, 1.4)), scope=int(f)) for f in scope])
+                for _ in range(count)]
+
+    def sums_over(left, right):
+        products = [Product(children=[a, b]) for a in left for b in right]
+        return [Sum(weights=[float(v) for v in rng.dirichlet(np.ones(len(products)))], children=products) for _ in range(8)]
+
+    def chain(scope, level):
+        na, nb_last = shapes[level]
+        left = leaves(scope[:2], na)
+        if level + 1 == len(shapes):
+            return sums_over(left, leaves(scope[2:], nb_last))
+        return sums_over(left, chain(scope[2:], level + 1))
+
+    def mirrored(scope, level):   # the same with the operands swapped: (8, na) groups
+        na, nb_last = shapes[level]
+        right = leaves(scope[:2], na)
+        if level + 1 == len(shapes):
+            return sums_over(leaves(scope[2:], nb_last), right)
+        return sums_over(mirrored(scope[2:], level + 1), right)
+
+    roots = chain(list(range(num_features)), 0) + mirrored(list(range(num_features))[::-1], 0)
+    spn = Sum(weights=[float(v) for v in rng.dirichlet(np.ones(len(roots)))], children=roots)
+    X = rng.normal(0, 1.2, (700, num_features))
+    if marginal:
+        X[rng.random(X.shape) < 0.2] = np.nan
+    return spn, X
+
+
+@pytest.mark.parametrize("case", [
+    ((2, 8), (4, 8), (8, 8), (4, 4)),        # groups of 2x8, 4x8, 8x8 and 4x4 products, and 8x2, 8x4, ... mirrored
+    ((4, 8), (2, 8), (8, 4)),
+    ((8, 8), (8, 8), (8, 8), (2, 8)),
+])
+@pytest.mark.parametrize("marginal", [False, True])
+def test_matrix_form_outer_sums(native, case, marginal):
+    """Every operand-count pair the matrix-core outer sum exists for, with slot lists in either tier."""
+    spn, X = _region_graph(77 + len(case), case, num_features=2 * len(case) + 2, marginal=marginal)
+    want64 = ev.ll_closed_f64(oracle_model(spn, "float64"), X, marginal=marginal)
+    # LDS limits below the program's slot count put the long-lived pool (tiered access) or any slot (select-the-base
+    # access) into the spill tier.
+    for opts in ({}, {"hip-interp-short-slots": 12, "hip-interp-lds-slots": 24},
+                 {"hip-interp-staged-features": "spill", "hip-interp-long-range": 4, "hip-interp-lds-slots": 24},
+                 {"hip-interp-short-slots": 12, "hip-interp-long-range": 2, "hip-interp-lds-slots": 20},
+                 {"hip-interp-matrix-core": "false"}, {"hip-interp-lds-slots": 6}):
+        k = compile_spn(native, spn, "float64", marginal=marginal, **dict(opts, **{"hip-kernel": "interpreter"}))
+        if opts.get("hip-interp-matrix-core") != "false":
+            assert "outersum(8 sums x" in k.source()
+        got = run(k, X)
+        assert got.dtype == np.float32
+        assert np.abs(got - want64).max() <= F32_TOL * max(1.0, np.abs(want64).max() / 100), opts
