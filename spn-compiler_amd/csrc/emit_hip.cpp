@@ -34,7 +34,7 @@ struct Emitter {
   Emitter(const Graph& graph, const CompileOptions& opts) : g(graph), o(opts) {
     logSpace = o.useLogSpace;
     f64 = !logSpace || o.computeType == ComputeType::F64;
-    log2Dom = logSpace && !f64 && o.log2Domain;
+    log2Dom = logSpace && o.log2Domain;  // float: hardware exp2/log2; double: the short routines emitted with the kernel
     scale = log2Dom ? 1.4426950408889634074 : 1.0;
   }
 
@@ -194,8 +194,12 @@ struct Emitter {
   // The log2-domain f32 kernel uses the hardware exp2/log2 instructions directly. The other
   // flavours call the accurate library routines through out-of-line wrappers: inlining them
   // thousands of times into one basic block makes register allocation take minutes.
-  std::string expOf(const std::string& a) const { return (log2Dom ? "__builtin_amdgcn_exp2f(" : "spn_exp(") + a + ")"; }
-  std::string logOf(const std::string& a) const { return (log2Dom ? "__builtin_amdgcn_logf(" : "spn_log(") + a + ")"; }
+  std::string expOf(const std::string& a) const {
+    return (log2Dom ? (f64 ? "spn_exp2(" : "__builtin_amdgcn_exp2f(") : "spn_exp(") + a + ")";
+  }
+  std::string logOf(const std::string& a) const {
+    return (log2Dom ? (f64 ? "spn_log2(" : "__builtin_amdgcn_logf(") : "spn_log(") + a + ")";
+  }
   std::string maxOf(const std::string& a, const std::string& b) const {
     return std::string(f64 ? "__builtin_fmax(" : "__builtin_fmaxf(") + a + ", " + b + ")";
   }
@@ -452,6 +456,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   if (!e.vectorRows) U = 1;
   js.samplesPerLane = U;
   js.libraryMath = !e.log2Dom;
+  js.doubleConstants = e.f64;
 
   std::ostringstream s;
   s << "// generated by spnc-hip for SPN '" << g.name << "': " << g.nodes.size() << " nodes, " << F << " features\n";
@@ -472,8 +477,40 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     s << "};\n";
   }
   // Out-of-line library math keeps hipRTC times in seconds for large graphs; small graphs inline it.
-  const bool inlineMath = g.nodes.size() + g.stats.sumTerms <= 4000;
+  const bool inlineMath = o.inlineMath >= 0 ? o.inlineMath == 1 : g.nodes.size() + g.stats.sumTerms <= 4000;
   const char* mathAttr = inlineMath ? "__forceinline__" : "__attribute__((noinline))";
+  if (e.log2Dom && e.f64) {
+    // Base-2 exponential and logarithm in double for the arguments this kernel produces (exponents <= 0 up to
+    // rounding, logarithms of sums in [1, fan-in] or of exactly 0): about 20 and 35 instructions where the
+    // general library routines take 40 and 95. exp2: 2^x = 2^n * 2^f, n = rint(x), |f| <= 1/2, 2^f by its Taylor
+    // series to degree 13 (remainder 4e-18). log2: x = 2^e * t, t in [sqrt(1/2), sqrt(2)), z = (t-1)/(t+1),
+    // log2 t = (2/ln 2) z (1 + z^2/3 + ... + z^18/19) (|z| <= 0.172, next term 2e-17). Both agree with the
+    // library to 5e-16 relative over their ranges (checked on the CPU against exp2/log2 of libm).
+    s << "static __device__ " << mathAttr << " real_t spn_exp2(real_t x) {\n"
+         "  x = x < -1100.0 ? -1100.0 : x;  // keeps NaN\n"
+         "  const real_t n = __builtin_rint(x), f = x - n;\n"
+         "  real_t p = 0x1.816193166d0f7p-40;\n"
+         "  p = __builtin_fma(p, f, 0x1.c3bd650fc2983p-36);\n  p = __builtin_fma(p, f, 0x1.e8cac7351bb22p-32);\n"
+         "  p = __builtin_fma(p, f, 0x1.e4cf5158b8ec7p-28);\n  p = __builtin_fma(p, f, 0x1.b5253d395e7c1p-24);\n"
+         "  p = __builtin_fma(p, f, 0x1.62c0223a5c822p-20);\n  p = __builtin_fma(p, f, 0x1.ffcbfc588b0c5p-17);\n"
+         "  p = __builtin_fma(p, f, 0x1.430912f86c786p-13);\n  p = __builtin_fma(p, f, 0x1.5d87fe78a6730p-10);\n"
+         "  p = __builtin_fma(p, f, 0x1.3b2ab6fba4e77p-7);\n  p = __builtin_fma(p, f, 0x1.c6b08d704a0bfp-5);\n"
+         "  p = __builtin_fma(p, f, 0x1.ebfbdff82c58ep-3);\n  p = __builtin_fma(p, f, 0x1.62e42fefa39efp-1);\n"
+         "  p = __builtin_fma(p, f, 1.0);\n"
+         "  return __builtin_ldexp(p, (int)n);\n}\n";
+    s << "static __device__ " << mathAttr << " real_t spn_log2(real_t x) {\n"
+         "  int e;\n  real_t t = __builtin_frexp(x, &e);\n"
+         "  const bool low = t < 0x1.6a09e667f3bcdp-1;\n  t = low ? t + t : t;\n  e = low ? e - 1 : e;\n"
+         "  const real_t z = (t - 1.0) / (t + 1.0), w = z * z;\n"
+         "  real_t p = 0x1.af286bca1af28p-5;\n"
+         "  p = __builtin_fma(p, w, 0x1.e1e1e1e1e1e1ep-5);\n  p = __builtin_fma(p, w, 0x1.1111111111111p-4);\n"
+         "  p = __builtin_fma(p, w, 0x1.3b13b13b13b14p-4);\n  p = __builtin_fma(p, w, 0x1.745d1745d1746p-4);\n"
+         "  p = __builtin_fma(p, w, 0x1.c71c71c71c71cp-4);\n  p = __builtin_fma(p, w, 0x1.2492492492492p-3);\n"
+         "  p = __builtin_fma(p, w, 0x1.999999999999ap-3);\n  p = __builtin_fma(p, w, 0x1.5555555555555p-2);\n"
+         "  p = __builtin_fma(p, w, 1.0);\n"
+         "  const real_t r = __builtin_fma(z * 0x1.71547652b82fep+1, p, (real_t)e);\n"
+         "  return x == 0.0 ? -__builtin_huge_val() : r;  // a sum whose terms are all impossible\n}\n";
+  }
   if (!e.log2Dom) {
     s << "static __device__ " << mathAttr << " real_t spn_exp(real_t x) { return " << (e.f64 ? "exp(x)" : "expf(x)") << "; }\n";
     s << "static __device__ " << mathAttr << " real_t spn_log(real_t x) { return " << (e.f64 ? "log(x)" : "logf(x)") << "; }\n";
@@ -481,7 +518,8 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   if (e.logSpace && o.sumForm == SumForm::Pairwise) {
     s << "static __device__ " << (e.log2Dom ? "__forceinline__" : mathAttr) << " real_t spn_logadd(real_t x, real_t y) {\n"
          "  const bool gt = x > y;\n  const real_t a = gt ? x : y;\n  const real_t b = gt ? y : x;\n";
-    if (e.f64) s << "  return a + log1p(exp(b - a));\n";
+    if (e.f64 && e.log2Dom) s << "  return a + spn_log2(1.0 + spn_exp2(b - a));\n";
+    else if (e.f64) s << "  return a + log1p(exp(b - a));\n";
     else if (e.log2Dom) s << "  return a + __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(b - a));\n";
     else s << "  return a + log1pf(expf(b - a));\n";
     s << "}\n";
@@ -520,7 +558,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   s << e.body.str();
   std::string root = Emitter::v(g.root());
   if (!e.logSpace) s << "  return spn_log(" << root << ");\n";
-  else if (e.log2Dom) s << "  return " << root << " * 0x1.62e43p-1f;\n";  // back to natural log: * ln 2
+  else if (e.log2Dom) s << "  return " << root << (e.f64 ? " * 0x1.62e42fefa39efp-1;\n" : " * 0x1.62e43p-1f;\n");  // back to natural log: * ln 2
   else s << "  return " << root << ";\n";
   s << "}\n";
 

@@ -21,7 +21,8 @@ struct JitSource {
   unsigned bytesPerResult = 4;
   unsigned tableEntries = 0;  // entries of the leaf-table pool (0 = none)
   bool tablesInLds = false;
-  bool libraryMath = false;   // calls ocml exp/log (float64, natural-log float32, linear space)
+  bool libraryMath = false;   // calls ocml exp/log (natural-log domain, linear space)
+  bool doubleConstants = false;  // computes in double: constants live in registers, not in instruction literals
   bool oneTilePerBlock = false;
   bool stagedInput = false;   // rows reach the lanes through an LDS tile ("gpu-shared-mem")
 };
