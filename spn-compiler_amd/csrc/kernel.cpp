@@ -23,7 +23,7 @@ void hipCheck(hipError_t e, const char* what) {
   if (e != hipSuccess) fatal(std::string("HIP error in ") + what + ": " + hipGetErrorString(e));
 }
 
-std::vector<char> compileWithHipRtc(const JitSource& js, int optLevel) {
+std::vector<char> compileWithHipRtc(const JitSource& js, int optLevel, int machineLicm) {
   hiprtcProgram prog;
   if (hiprtcCreateProgram(&prog, js.source.c_str(), "spn_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
     fatal("hiprtcCreateProgram failed");
@@ -34,7 +34,7 @@ std::vector<char> compileWithHipRtc(const JitSource& js, int optLevel) {
   // The kernel body sits in a grid-stride loop. Double constants cannot be instruction literals, and machine LICM
   // moves the thousands of register moves that materialise them out of that loop, where they no longer fit the
   // register file (measured on a 1389-node graph: 512 VGPRs plus 1612 spills with it, 75 VGPRs without).
-  if (js.doubleConstants) {
+  if (machineLicm == 0 || (machineLicm < 0 && js.doubleConstants)) {
     opts.push_back("-mllvm");
     opts.push_back("-disable-machine-licm");
   }
@@ -161,7 +161,7 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
     // optimiser stretches live ranges until the float64 kernels spill (512 VGPRs plus scratch,
     // about 7x slower on the 16-feature Gaussian tree).
     const int level = (js.libraryMath && !o.optLevelGiven) ? 1 : o.optLevel;
-    k->codeObject_ = compileWithHipRtc(js, level);
+    k->codeObject_ = compileWithHipRtc(js, level, o.machineLicm);
     k->entry_ = js.entry;
     k->blockSize_ = js.blockSize;
     k->samplesPerLane_ = js.samplesPerLane;

@@ -106,6 +106,8 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
     } else if (key == "hip-interp-long-range") {
       o.interpLongRange = parseInt(key, val);
       if (o.interpLongRange < -1) throw std::runtime_error("hip-interp-long-range must be -1 or a count of instructions");
+    } else if (key == "hip-machine-licm") {
+      o.machineLicm = val == "auto" ? -1 : (parseBool(val) ? 1 : 0);
     } else if (key == "hip-inline-math") {
       o.inlineMath = val == "auto" ? -1 : (parseBool(val) ? 1 : 0);
     } else if (key == "hip-table-budget-kib") {

@@ -34,6 +34,7 @@ struct CompileOptions {
   bool nontemporalLoads = true;                // "hip-nontemporal-loads": mark input loads as streaming
   bool eagerIndices = true;                    // "hip-eager-indices": compute table indices of all features first
   bool jointTables = true;                     // "hip-joint-tables": pair table leaves of a product into joint tables
+  int machineLicm = -1;                        // "hip-machine-licm": machine LICM on (1), off (0) or off for double kernels only (-1)
   int inlineMath = -1;                         // "hip-inline-math": exp/log routines inlined (1), called (0) or decided by graph size (-1)
   int tableBudgetKiB = 62;                     // "hip-table-budget-kib": LDS the table pool may grow to when leaves are paired into joint tables
   int jointMaxEntries = 160;                   // "hip-joint-max-entries": largest joint table (entries) a pair of table leaves may get
