@@ -284,8 +284,9 @@ template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB>
 __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
   typedef Math<float, LOG2> Mt;
   constexpr int M = 8, K = NA * NB, GROUPS = K / 16;
-  constexpr int DST = 3, AS = DST + M, BS = AS + NA;  // positions in the head: length, opcode, M, then the slot lists
-  static_assert(BS + NB <= Head::WORDS, "the slot lists must lie within the prefetched head");
+  // Positions in the head: length, opcode, M and format, then the slot lists and the three scale slots.
+  constexpr int DST = 3, AS = DST + M, BS = AS + NA, SCALES = BS + NB;
+  static_assert(SCALES + 3 <= Head::WORDS, "the slot lists must lie within the prefetched head");
   float A[GROUPS][2];
   const float* wl = wGlobal + (threadIdx.x & 63u);
 #pragma unroll
@@ -293,13 +294,13 @@ __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, c
     A[g][0] = wl[g * 128];
     A[g][1] = wl[g * 128 + 64];
   }
+  const uint32_t w0 = h.word(1);
+  const bool aScaled = (w0 >> 30) & 1u, bScaled = (w0 >> 31) & 1u, outScaled = (h.word(2) >> 8) & 1u;
   float ea[NA], eb[NB];
-  float ma = -__builtin_huge_valf(), mb = -__builtin_huge_valf();
   // Flagged instructions: the tier bits say per slot list where it lives (valid when exactly the short pool is
   // in LDS), so a list is read with LDS instructions or with scalar-base global loads; mixed lists and other
   // LDS splits take the select-the-base form.
-  const uint32_t tierA = TIERED ? (h.word(1) >> 24) & 3u : 2u, tierB = TIERED ? (h.word(1) >> 26) & 3u : 2u,
-                 tierD = TIERED ? (h.word(1) >> 28) & 3u : 2u;
+  const uint32_t tierA = TIERED ? (w0 >> 24) & 3u : 2u, tierB = TIERED ? (w0 >> 26) & 3u : 2u, tierD = TIERED ? (w0 >> 28) & 3u : 2u;
   if (!SPILL || tierA == 0) {
 #pragma unroll
     for (int r = 0; r < NA; ++r) ea[r] = S.rdLds(h.word(AS + r));
@@ -320,24 +321,51 @@ __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, c
 #pragma unroll
     for (int c = 0; c < NB; ++c) eb[c] = S.rd(h.word(BS + c));
   }
+  // A scaled list already holds exp2(value - max) and brings max along in its scale slot; a list of log2
+  // values is shifted by its maximum and exponentiated here. All slots are read before any is written.
+  float base = 0.f;
+  if (aScaled) {
+    base += S.rd(h.word(SCALES + 1));
+  } else {
+    float ma = -__builtin_huge_valf();
 #pragma unroll
-  for (int r = 0; r < NA; ++r) ma = rmax(ma, ea[r]);
+    for (int r = 0; r < NA; ++r) ma = rmax(ma, ea[r]);
+    ma = rmax(ma, Mt::lowest());
 #pragma unroll
-  for (int c = 0; c < NB; ++c) mb = rmax(mb, eb[c]);
-  ma = rmax(ma, Mt::lowest());
-  mb = rmax(mb, Mt::lowest());
+    for (int r = 0; r < NA; ++r) ea[r] = Mt::exp(ea[r] - ma);
+    base += ma;
+  }
+  if (bScaled) {
+    base += S.rd(h.word(SCALES + 2));
+  } else {
+    float mb = -__builtin_huge_valf();
 #pragma unroll
-  for (int r = 0; r < NA; ++r) ea[r] = Mt::exp(ea[r] - ma);
+    for (int c = 0; c < NB; ++c) mb = rmax(mb, eb[c]);
+    mb = rmax(mb, Mt::lowest());
 #pragma unroll
-  for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(eb[c] - mb);
+    for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(eb[c] - mb);
+    base += mb;
+  }
   float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
   MatrixSteps<0, K, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
-  const float base = ma + mb;
   float res[M];
+  if (outScaled) {
+    // acc_t / max(acc) and one logarithm for the whole vector. All-zero accumulators (impossible evidence) give
+    // zeros and a scale of -inf; the floor under the maximum only keeps the reciprocal finite.
+    float m = rmax(rmax(rmax(d0[0], d0[1]), rmax(d0[2], d0[3])), rmax(rmax(d1[0], d1[1]), rmax(d1[2], d1[3])));
+    const float inv = __builtin_amdgcn_rcpf(rmax(m, 0x1p-100f));
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    res[t] = base + Mt::log(d0[t]);
-    res[4 + t] = base + Mt::log(d1[t]);
+    for (int t = 0; t < 4; ++t) {
+      res[t] = d0[t] * inv;
+      res[4 + t] = d1[t] * inv;
+    }
+    S.wr(h.word(SCALES), base + Mt::log(m));
+  } else {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      res[t] = base + Mt::log(d0[t]);
+      res[4 + t] = base + Mt::log(d1[t]);
+    }
   }
   if (!SPILL || tierD == 0) {
 #pragma unroll
@@ -349,7 +377,7 @@ __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, c
 #pragma unroll
     for (int t = 0; t < M; ++t) S.wr(h.word(DST + t), res[t]);
   }
-  return ip + 2 + M + NA + NB + K * M;
+  return ip + 2 + M + NA + NB + 3 + K * M;
 }
 
 // The operand counts the program builder emits the matrix form for (matrixFormShape in interp_program.cpp).
@@ -504,8 +532,8 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
   const int na = int((w0 >> 8) & 0xffu), nb = int((w0 >> 16) & 0xffu);
   if constexpr (sizeof(R) == 4) {
     if (op == OP_OUTERMM) {
-      // The weights start after the two header words, eight destinations and na + nb operands.
-      const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 10 + na + nb);
+      // The weights start after the two header words, eight destinations, na + nb operands and three scale slots.
+      const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 13 + na + nb);
       return outerSumMatrixAny<LOG2, SPILL, TIERED>(ip, h, na, nb, wGlobal, S);
     }
   }

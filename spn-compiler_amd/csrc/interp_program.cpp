@@ -65,16 +65,16 @@ bool matrixFormShape(uint32_t na, uint32_t nb) {
 // short pool fits the LDS share that lets four blocks reside on a CU, or failing that two.
 InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
   const bool f64 = o.computeType == ComputeType::F64;
-  // Short-pool sizes (slots of 256 values) that let six, four or two blocks share the 160 KiB of a CU.
-  const uint32_t sixBlocks = o.interpShortSlots > 0 ? uint32_t(o.interpShortSlots) : (f64 ? 13 : 26), fourBlocks = f64 ? 20 : 40,
+  // Short-pool sizes (slots of 256 values) that let five or six, four, or two blocks share the 160 KiB of a CU.
+  const uint32_t manyBlocks = o.interpShortSlots > 0 ? uint32_t(o.interpShortSlots) : (f64 ? 13 : 27), fourBlocks = f64 ? 20 : 40,
                  twoBlocks = f64 ? 36 : 72;
   // Candidates differ in which values count as long-lived (and so may leave LDS) and in the tier of
-  // the staged features. Preferred: the most blocks per CU (measured on a RAT-SPN: 9.0 ms with six,
-  // 9.7 ms with four, 10.1 ms with eight blocks of 16 slots); among equals the candidate that
-  // touches the spill tier least.
+  // the staged features. Preferred: five or six blocks per CU (measured on a RAT-SPN: 8.8 ms with
+  // pools of 24 to 27 slots, 9.4 ms with 36 or 40, 9.4 to 10.1 ms with 16 to 20 slots and eight
+  // blocks); among equals the candidate that touches the spill tier least.
   InterpProgram best;
   bool have = false;
-  auto rank = [&](const InterpProgram& p) { return p.shortSlots <= sixBlocks ? 0 : (p.shortSlots <= fourBlocks ? 1 : (p.shortSlots <= twoBlocks ? 2 : 3)); };
+  auto rank = [&](const InterpProgram& p) { return p.shortSlots <= manyBlocks ? 0 : (p.shortSlots <= fourBlocks ? 1 : (p.shortSlots <= twoBlocks ? 2 : 3)); };
   auto better = [&](const InterpProgram& p) {
     if (!have) return true;
     const int rp = rank(p), rb = rank(best);
@@ -274,6 +274,42 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
     instrs.push_back(std::move(in));
   }
 
+  // ---- matrix-form outer sums and the format of the vectors between them ----
+  // An outer sum in matrix form whose eight results are read by exactly one other such instruction, as its
+  // complete a or b list, hands them over as a scaled linear vector: acc_t / max(acc) in the eight slots and
+  // one more slot holding the common log2 scale. The consumer then needs no maximum, subtraction or
+  // exponential for that list and the producer one logarithm instead of eight.
+  std::vector<bool> matrixInstr(instrs.size(), false);
+  std::vector<int> linearConsumer(instrs.size(), -1);  // producer -> consuming instruction
+  {
+    for (uint32_t k = 0; k < instrs.size(); ++k) {
+      const Instr& in = instrs[k];
+      if (in.op != OP_OUTERSUM) continue;
+      const Outer& outer = outerOf.at(g.nodes[in.node].children);
+      matrixInstr[k] = !p.f64 && in.defs.size() == 8 && o.interpMatrixCore &&
+                       matrixFormShape(uint32_t(outer.a.size()), uint32_t(outer.b.size()));
+    }
+    std::vector<std::vector<uint32_t>> readers(N);
+    for (uint32_t k = 0; k < instrs.size(); ++k)
+      for (uint32_t sidx : instrs[k].srcs)
+        if (readers[sidx].empty() || readers[sidx].back() != k) readers[sidx].push_back(k);
+    for (uint32_t k = 0; k < instrs.size() && o.interpScaledVectors; ++k) {
+      if (!matrixInstr[k]) continue;
+      const Instr& in = instrs[k];
+      int consumer = -1;
+      bool ok = true;
+      for (uint32_t d : in.defs) {
+        if (d == g.root() || readers[d].size() != 1) ok = false;
+        else if (consumer < 0) consumer = int(readers[d][0]);
+        else if (consumer != int(readers[d][0])) ok = false;
+      }
+      if (!ok || consumer < 0 || !matrixInstr[consumer]) continue;
+      const Outer& co = outerOf.at(g.nodes[instrs[consumer].node].children);
+      if (co.a == in.defs || co.b == in.defs) linearConsumer[k] = consumer;
+    }
+  }
+  std::vector<uint32_t> scaleSlotOfNode(N, NONE);  // first result of a scaled linear vector -> slot of its scale
+
   // ---- slot allocation by liveness on the instruction order ----
   std::vector<uint32_t> lastUse(N, 0);
   for (uint32_t k = 0; k < instrs.size(); ++k)
@@ -371,7 +407,10 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       std::sort(uniq.begin(), uniq.end());
       uniq.erase(std::unique(uniq.begin(), uniq.end()), uniq.end());
       for (uint32_t s : uniq)
-        if (lastUse[s] == k) releaseSlot(slotOf[s]);
+        if (lastUse[s] == k) {
+          releaseSlot(slotOf[s]);
+          if (scaleSlotOfNode[s] != NONE) releaseSlot(scaleSlotOfNode[s]);
+        }
     }
     for (uint32_t d : in.defs) slotOf[d] = allocSlot(d);
     // Bit 7 of the opcode tells the kernel that this instruction touches the long pool.
@@ -438,21 +477,39 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
         // A single leftover sum is encoded as a layer of two identical sums writing the same slot.
         std::vector<uint32_t> defs = in.defs;
         if (m == 1) defs.push_back(in.defs[0]);
-        const bool matrixForm = !p.f64 && defs.size() == 8 && o.interpMatrixCore && matrixFormShape(na, nb);
+        const bool matrixForm = matrixInstr[k];
         const size_t at = b.begin();
         // Matrix form: bits 24-29 say where each slot list lives (0 all in the short pool, 1 all in the long pool,
-        // 2 mixed), so the kernel picks the access instructions per list, not per slot.
+        // 2 mixed), so the kernel picks the access instructions per list, not per slot; bits 30 and 31 say that
+        // the a / b list is a scaled linear vector; bit 8 of the second word that the result is one.
         auto tierOf = [&](const std::vector<uint32_t>& nodes) {
           uint32_t longOnes = 0;
           for (uint32_t x : nodes) longOnes += (slotOf[x] & LONG_BIT) ? 1 : 0;
           return longOnes == 0 ? 0u : (longOnes == nodes.size() ? 1u : 2u);
         };
-        const uint32_t tiers = matrixForm ? (tierOf(outer.a) << 24) | (tierOf(outer.b) << 26) | (tierOf(defs) << 28) : 0u;
+        const uint32_t scaleA = matrixForm ? scaleSlotOfNode[outer.a[0]] : NONE, scaleB = matrixForm ? scaleSlotOfNode[outer.b[0]] : NONE;
+        uint32_t scaleDst = NONE;
+        if (matrixForm && linearConsumer[k] >= 0) {
+          scaleDst = allocSlot(in.defs[0]);  // lives exactly as long as the vector
+          scaleSlotOfNode[in.defs[0]] = scaleDst;
+          if (scaleDst & LONG_BIT) longFlag |= 0x80u;
+        }
+        if (scaleA != NONE && (scaleA & LONG_BIT)) longFlag |= 0x80u;
+        if (scaleB != NONE && (scaleB & LONG_BIT)) longFlag |= 0x80u;
+        const uint32_t tiers = matrixForm ? (tierOf(outer.a) << 24) | (tierOf(outer.b) << 26) | (tierOf(defs) << 28) |
+                                                (scaleA != NONE ? 1u << 30 : 0u) | (scaleB != NONE ? 1u << 31 : 0u)
+                                          : 0u;
         b.word((matrixForm ? OP_OUTERMM : OP_OUTERSUM) | longFlag | (na << 8) | (nb << 16) | tiers);
-        b.word(uint32_t(defs.size()));
+        b.word(uint32_t(defs.size()) | (scaleDst != NONE ? 0x100u : 0u));
         for (uint32_t d : defs) slotWord(slotOf[d]);
         for (uint32_t a : outer.a) slotWord(slotOf[a]);
         for (uint32_t c : outer.b) slotWord(slotOf[c]);
+        if (matrixForm) {  // the three scale slots, unused ones as NONE
+          for (uint32_t sc : {scaleDst, scaleA, scaleB}) {
+            if (sc != NONE) slotWord(sc);
+            else b.word(NONE);
+          }
+        }
         if (matrixForm) {
           for (uint32_t grp = 0; grp < na * nb / 16; ++grp)
             for (uint32_t half = 0; half < 2; ++half)
@@ -462,8 +519,8 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
             for (uint32_t d : defs) b.real(g.nodes[d].weights[j]);
         }
         b.end(at);
-        b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = outersum(" << m << " sums x " << na << "x" << nb << " products)   ; nodes " << in.defs[0]
-              << "..\n";
+        b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = outersum(" << m << " sums x " << na << "x" << nb << " products)"
+              << (scaleDst != NONE ? " scaled" : "") << "   ; nodes " << in.defs[0] << "..\n";
         break;
       }
       default:

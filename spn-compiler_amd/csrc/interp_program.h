@@ -25,8 +25,12 @@ enum InterpOp : uint32_t {
   OP_SUMLAYER = 3,  // [op|k<<8][M][dst*M] k*slot, k*M weights        M sums over the same k children (M in 2,4,8)
   OP_OUTERSUM = 4,  // [op|NA<<8|NB<<16][M][dst*M] NA*slot, NB*slot, NA*NB*M weights
                     //   M sums over all products a_r * b_c of two operand vectors, products never materialised
-  OP_OUTERMM = 6,   // [op|NA<<8|NB<<16|tiers<<24][8][dst*8] NA*slot, NB*slot, NA*NB*8 weights in matrix-core order
+  OP_OUTERMM = 6,   // [op|NA<<8|NB<<16|tiers<<24|aScaled<<30|bScaled<<31][8|outScaled<<8][dst*8] NA*slot, NB*slot,
+                    //   [scale slot of dst, of a, of b (0xFFFFFFFF where unused)], NA*NB*8 weights in matrix-core order
                     //   tiers: two bits each for the a, b and dst lists: 0 all short-pool slots, 1 all long-pool, 2 mixed
+                    //   A scaled list holds v_i / max(v) (linear, in [0,1]) and its scale slot log2 max(v) plus the
+                    //   scales it inherited: value_i = scale + log2(slot_i). Such vectors only travel between
+                    //   matrix-form outer sums; they save the consumer's exponentials and the producer's logarithms.
                     //   OUTERSUM for float, eight sums and NA*NB a multiple of 16: weight of product k = r*NB + c and
                     //   sum t sits at word (k/16)*128 + (t/4)*64 + (k%16)*4 + t%4, i.e. 64-word rows that one
                     //   wavefront loads with one coalesced access and that feed sixteen 4x4x1 matrix instructions

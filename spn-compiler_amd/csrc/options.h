@@ -34,11 +34,12 @@ struct CompileOptions {
   bool nontemporalLoads = true;                // "hip-nontemporal-loads": mark input loads as streaming
   bool eagerIndices = true;                    // "hip-eager-indices": compute table indices of all features first
   bool jointTables = true;                     // "hip-joint-tables": pair table leaves of a product into joint tables
-  int machineLicm = -1;                        // "hip-machine-licm": machine LICM on (1), off (0) or off for double kernels only (-1)
+  int machineLicm = -1;                        // "hip-machine-licm": machine LICM for generated kernels on (1), off (0) or decided per kernel (-1)
   int inlineMath = -1;                         // "hip-inline-math": exp/log routines inlined (1), called (0) or decided by graph size (-1)
   int tableBudgetKiB = 62;                     // "hip-table-budget-kib": LDS the table pool may grow to when leaves are paired into joint tables
   int jointMaxEntries = 160;                   // "hip-joint-max-entries": largest joint table (entries) a pair of table leaves may get
   int interpShortSlots = 0;                    // "hip-interp-short-slots": LDS value slots per lane the interpreter program aims for (0 = automatic)
+  bool interpScaledVectors = true;             // "hip-interp-scaled-vectors": region vectors between matrix-form outer sums travel as scaled linear values
   bool interpMatrixCore = true;                // "hip-interp-matrix-core": float outer sums of eight sums run on the matrix cores
   int interpLdsSlots = 0;                      // "hip-interp-lds-slots": upper bound on the value slots the launcher keeps in LDS (0 = automatic)
   int interpStagedLong = -1;                   // "hip-interp-staged-features": lds|spill (-1 = automatic): tier of the staged input features

@@ -351,12 +351,23 @@ Graph buildGraph(const RawQuery& q) {
   // [prod(a_0,b_0), ..., prod(a_NA-1,b_NB-1)] and nothing else reads those products. Since
   // exp(a_r + b_c - ma - mb) = exp(a_r - ma) * exp(b_c - mb), the group costs NA + NB exponentials, not M*NA*NB.
   // Where that factored form is cheaper than the per-sum accounting above, it is the algorithmic minimum.
-  std::map<std::vector<uint32_t>, uint64_t> groups;
-  for (const auto& n : g.nodes)
-    if (n.kind == NodeKind::Sum && n.children.size() >= 4) groups[n.children]++;
-  for (const auto& entry : groups) {
+  // A group whose sums are read only by the products of one other group, as that group's complete first or
+  // second operand vector, can hand them over as acc_t / max(acc) plus one common scale: one logarithm and one
+  // reciprocal for the vector instead of a logarithm per sum, and no maximum, shift or exponential for that
+  // vector in the consumer.
+  struct OuterGroup {
+    std::vector<uint32_t> members, a, b;  // the sums (ascending node order) and the two operand vectors
+    uint64_t k = 0;
+    bool outScaled = false, aScaled = false, bScaled = false;
+  };
+  std::map<std::vector<uint32_t>, std::vector<uint32_t>> byChildren;
+  for (uint32_t i = 0; i < g.nodes.size(); ++i)
+    if (g.nodes[i].kind == NodeKind::Sum && g.nodes[i].children.size() >= 4) byChildren[g.nodes[i].children].push_back(i);
+  std::vector<OuterGroup> outerGroups;
+  std::vector<int> groupOfProduct(g.nodes.size(), -1);
+  for (const auto& entry : byChildren) {
     const std::vector<uint32_t>& kids = entry.first;
-    const uint64_t members = entry.second, k = kids.size();
+    const uint64_t members = entry.second.size(), k = kids.size();
     bool ok = true;
     for (uint32_t c : kids) {
       const auto& pn = g.nodes[c];
@@ -376,11 +387,47 @@ Graph buildGraph(const RawQuery& q) {
     std::sort(sorted.begin(), sorted.end());
     if (std::adjacent_find(sorted.begin(), sorted.end()) != sorted.end()) ok = false;
     if (!ok) continue;
+    OuterGroup og;
+    og.members = entry.second;
+    og.k = k;
+    for (uint64_t r = 0; r < na; ++r) og.a.push_back(g.nodes[kids[r * nb]].children[0]);
+    for (uint64_t c = 0; c < nb; ++c) og.b.push_back(g.nodes[kids[c]].children[1]);
+    for (uint32_t c : kids) groupOfProduct[c] = int(outerGroups.size());
+    outerGroups.push_back(std::move(og));
+  }
+  std::vector<std::vector<uint32_t>> parents(g.nodes.size());
+  for (uint32_t i = 0; i < g.nodes.size(); ++i)
+    for (uint32_t c : g.nodes[i].children) parents[c].push_back(i);
+  for (auto& og : outerGroups) {
+    int consumer = -1;
+    bool ok = true;
+    for (uint32_t m : og.members) {
+      if (m == g.root() || parents[m].empty()) ok = false;
+      for (uint32_t pa : parents[m]) {
+        if (groupOfProduct[pa] < 0) ok = false;
+        else if (consumer < 0) consumer = groupOfProduct[pa];
+        else if (consumer != groupOfProduct[pa]) ok = false;
+      }
+    }
+    if (!ok || consumer < 0) continue;
+    OuterGroup& cg = outerGroups[size_t(consumer)];
+    if (cg.a == og.members) cg.aScaled = og.outScaled = true;
+    else if (cg.b == og.members) cg.bScaled = og.outScaled = true;
+  }
+  for (const auto& og : outerGroups) {
+    const uint64_t members = og.members.size(), k = og.k, na = og.a.size(), nb = og.b.size();
     // Per-sum accounting of the group, products included (k >= 4, so the n-ary form was the one charged).
     const uint64_t naiveFlops = members * 5 * k + k, naiveTrans = members * (k + 1);
-    // Factored: two maxima and shifts (2 per operand), NA*NB products of exponentials, M*NA*NB multiply-adds,
-    // a logarithm and two adds per sum.
-    const uint64_t factFlops = 2 * (na + nb) + k + members * k + 2 * members, factTrans = na + nb + members;
+    // Factored: per log-valued operand vector a maximum, a shift and an exponential per element (a scaled one
+    // costs one add for its scale); NA*NB products; M*NA*NB multiply-adds; then a logarithm and an add per sum,
+    // or for a scaled result M-1 maxima, a reciprocal, M multiplies, one logarithm and one add.
+    uint64_t factFlops = k + members * k, factTrans = 0;
+    factFlops += og.aScaled ? 1 : 2 * na;
+    factTrans += og.aScaled ? 0 : na;
+    factFlops += og.bScaled ? 1 : 2 * nb;
+    factTrans += og.bScaled ? 0 : nb;
+    factFlops += og.outScaled ? (members - 1) + members + 1 : 2 * members;
+    factTrans += og.outScaled ? 2 : members;
     if (factFlops + 3 * factTrans < naiveFlops + 3 * naiveTrans) {
       st.flopsMin = st.flopsMin - naiveFlops + factFlops;
       st.transMin = st.transMin - naiveTrans + factTrans;

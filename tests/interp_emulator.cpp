@@ -137,33 +137,57 @@ int main(int argc, char** argv) {
           for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), m + lg(res[t]));
           pc = w + size_t(k) * M;
         } else if (op == OP_OUTERSUM || op == OP_OUTERMM) {
-          const uint32_t na = (w0 >> 8) & 0xff, nb = (w0 >> 16) & 0xff, M = c.at(pc + 1);
-          if (op == OP_OUTERMM) {  // the tier bits must describe the slot lists
-            auto tier = [&](size_t first, uint32_t count) {
+          const bool mm = op == OP_OUTERMM;
+          const uint32_t na = (w0 >> 8) & 0xff, nb = (w0 >> 16) & 0xff, M = c.at(pc + 1) & 0xff;
+          const size_t d0 = pc + 2, a0 = d0 + M, b0 = a0 + na, sc = b0 + nb, w = sc + (mm ? 3 : 0);
+          const bool aScaled = mm && ((w0 >> 30) & 1), bScaled = mm && ((w0 >> 31) & 1), outScaled = mm && ((c.at(pc + 1) >> 8) & 1);
+          if (mm) {
+            if (M != 8 || (na * nb) % 16 != 0) throw std::runtime_error("malformed matrix-form outer sum at word " + std::to_string(pc));
+            auto tier = [&](size_t first, uint32_t count) {  // the tier bits must describe the slot lists
               uint32_t longOnes = 0;
               for (uint32_t j = 0; j < count; ++j) longOnes += c.at(first + j) >= p.shortSlots ? 1 : 0;
               return longOnes == 0 ? 0u : (longOnes == count ? 1u : 2u);
             };
-            const uint32_t want = (tier(pc + 2 + M, na) << 24) | (tier(pc + 2 + M + na, nb) << 26) | (tier(pc + 2, M) << 28);
+            const uint32_t want = (tier(a0, na) << 24) | (tier(b0, nb) << 26) | (tier(d0, M) << 28);
             if ((w0 & 0x3f000000u) != want) throw std::runtime_error("tier bits disagree with the slot lists at word " + std::to_string(pc));
+            if ((c.at(sc) != UINT32_MAX) != outScaled || (c.at(sc + 1) != UINT32_MAX) != aScaled || (c.at(sc + 2) != UINT32_MAX) != bScaled)
+              throw std::runtime_error("scale slots disagree with the format bits at word " + std::to_string(pc));
           }
-          if (op == OP_OUTERMM && (M != 8 || (na * nb) % 16 != 0)) throw std::runtime_error("malformed matrix-form outer sum at word " + std::to_string(pc));
           // Matrix form: product k and sum t at (k/16)*128 + (t/4)*64 + (k%16)*4 + t%4.
-          auto weightAt = [&](size_t w, uint32_t k, uint32_t t) {
-            return asFloat(op == OP_OUTERMM ? c.at(w + (k / 16) * 128 + (t / 4) * 64 + (k % 16) * 4 + t % 4) : c.at(w + size_t(k) * M + t));
+          auto weightAt = [&](uint32_t k, uint32_t t) {
+            return asFloat(mm ? c.at(w + (k / 16) * 128 + (t / 4) * 64 + (k % 16) * 4 + t % 4) : c.at(w + size_t(k) * M + t));
           };
-          const size_t d0 = pc + 2, a0 = d0 + M, b0 = a0 + na, w = b0 + nb;
-          float ma = -INFINITY, mb = -INFINITY;
-          for (uint32_t r = 0; r < na; ++r) ma = std::fmax(ma, rd(c.at(a0 + r)));
-          for (uint32_t cc = 0; cc < nb; ++cc) mb = std::fmax(mb, rd(c.at(b0 + cc)));
-          ma = std::fmax(ma, -3.4028234663852886e38f);
-          mb = std::fmax(mb, -3.4028234663852886e38f);
+          // Operand vectors as exp2(value - max) plus the max (a scaled list is stored that way, its max in the scale slot).
+          auto operand = [&](size_t first, uint32_t count, bool scaled, size_t scaleAt, std::vector<float>& e) {
+            e.resize(count);
+            if (scaled) {
+              for (uint32_t j = 0; j < count; ++j) {
+                e[j] = rd(c.at(first + j));
+                if (!(e[j] >= 0.f && e[j] <= 1.0001f)) throw std::runtime_error("scaled operand outside [0,1] at word " + std::to_string(pc));
+              }
+              return rd(c.at(scaleAt));
+            }
+            float m = -INFINITY;
+            for (uint32_t j = 0; j < count; ++j) m = std::fmax(m, rd(c.at(first + j)));
+            m = std::fmax(m, -3.4028234663852886e38f);
+            for (uint32_t j = 0; j < count; ++j) e[j] = ex(rd(c.at(first + j)) - m);
+            return m;
+          };
+          std::vector<float> ea, eb;
+          const float base = operand(a0, na, aScaled, sc + 1, ea) + operand(b0, nb, bScaled, sc + 2, eb);
           std::vector<float> res(M, 0.f);
           for (uint32_t t = 0; t < M; ++t)
             for (uint32_t r = 0; r < na; ++r)
-              for (uint32_t cc = 0; cc < nb; ++cc)
-                res[t] += ex(rd(c.at(a0 + r)) - ma) * ex(rd(c.at(b0 + cc)) - mb) * weightAt(w, r * nb + cc, t);
-          for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), ma + mb + lg(res[t]));
+              for (uint32_t cc = 0; cc < nb; ++cc) res[t] += ea[r] * eb[cc] * weightAt(r * nb + cc, t);
+          if (outScaled) {
+            float m = 0.f;
+            for (uint32_t t = 0; t < M; ++t) m = std::fmax(m, res[t]);
+            const float inv = 1.0f / std::fmax(m, 0x1p-100f);
+            for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), res[t] * inv);
+            wr(c.at(sc), base + lg(m));
+          } else {
+            for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), base + lg(res[t]));
+          }
           pc = w + size_t(na) * nb * M;
         } else {
           throw std::runtime_error("unknown opcode at word " + std::to_string(pc));

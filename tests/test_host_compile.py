@@ -200,7 +200,12 @@ def test_generated_source_variants(native):
     os.remove(k.fileName())
     # the program builder honours the tier and pool-size options
     k = compile_spn(native, syn.c4_spn(), "float32", **{"hip-interp-staged-features": "lds", "hip-interp-long-range": 8, "hip-interp-short-slots": 40})
-    assert "136 value slots (32 staged features, 96 long-lived)" in k.source()
+    assert "140 value slots (32 staged features, 99 long-lived)" in k.source()   # 41 = 32 features + one vector of 8 and its scale
+    assert k.source().count(") scaled ") == 140             # every region vector that only feeds another region
+    os.remove(k.fileName())
+    k = compile_spn(native, syn.c4_spn(), "float32", **{"hip-interp-scaled-vectors": "false", "hip-interp-staged-features": "lds",
+                                                        "hip-interp-long-range": 8, "hip-interp-short-slots": 40})
+    assert "136 value slots (32 staged features, 96 long-lived)" in k.source() and ") scaled " not in k.source()
     os.remove(k.fileName())
 
 
