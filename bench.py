@@ -27,11 +27,11 @@ FP64_VECTOR_PEAK_TFLOPS = 78.6   # MI355X FP64 vector, published
 # workload -> (samples per launch, bytes). Only valid for that launch size and the default options.
 MEASURED_HBM_TRAFFIC = {
     "c1": (67108864, 1879038976),
-    "c2": (16777216, 1142135777),
-    "c3": (8388608, 3495408948),
-    "c4": (4194304, 10921959036),
-    "c5": (16777216, 1141495178),
-    "c5_f64": (16777216, 1212272946),
+    "c2": (16777216, 1142124104),
+    "c3": (8388608, 3495407719),
+    "c4": (4194304, 11090027198),
+    "c5": (16777216, 1141489649),
+    "c5_f64": (16777216, 1210438801),
 }
 
 
