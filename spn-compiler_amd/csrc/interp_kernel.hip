@@ -261,7 +261,10 @@ struct MatrixSteps {
             : "+v"(d0), "+v"(d1), "=&v"(e2)
             : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "v"(ea[(K + 2) / NB]), "v"(eb[(K + 2) % NB]), "n"(K % 16), "v"(e1));
       } else {
+        // The leading s_nop separates the first matrix instruction from a register copy the compiler might place
+        // between two statements (it cannot know that the statement opens with a matrix instruction).
         asm volatile(
+            "s_nop 0\n\t"
             "v_mfma_f32_4x4x1_16b_f32 %0, %3, %5, %0 cbsz:4 abid:%8\n\t"
             "v_mul_f32 %2, %6, %7\n\t"
             "v_mfma_f32_4x4x1_16b_f32 %1, %4, %5, %1 cbsz:4 abid:%8"
@@ -271,6 +274,7 @@ struct MatrixSteps {
       MatrixSteps<K + 1, KEND, NB>::run(ea, eb, A, d0, d1, e1, e2);
     } else {
       asm volatile(
+          "s_nop 0\n\t"
           "v_mfma_f32_4x4x1_16b_f32 %0, %2, %4, %0 cbsz:4 abid:%5\n\t"
           "v_mfma_f32_4x4x1_16b_f32 %1, %3, %4, %1 cbsz:4 abid:%5"
           : "+v"(d0), "+v"(d1)

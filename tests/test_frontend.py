@@ -125,3 +125,12 @@ def test_cpu_baseline_kernel_follows_the_oracle(tmp_path):
         so, _ = cgen.build(m, marginal, workdir=str(tmp_path / dtype))
         got = cgen.load(so, dtype)(X)
         assert np.abs(got - ev.ll_reforder(m, X, np.float32, marginal=marginal)).max() < 2e-6
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU; asking for more exits with a message instead of a number."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in (r.stdout + r.stderr)
