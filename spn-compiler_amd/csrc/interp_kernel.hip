@@ -248,11 +248,14 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 // matrix result are held back by the hardware.
 template <int K, int KEND, int NB>
 struct MatrixSteps {
+  // e: product of this step, e1: product of the next step (made one step ago, used one step from now).
   static __device__ __forceinline__ void run(const float* ea, const float* eb, const float (*A)[2], float4v& d0, float4v& d1, float e,
                                              float e1) {
     if constexpr (K + 2 < KEND) {
       float e2;
       if constexpr (K == 0) {
+        // The two wait states in front separate the first matrix instruction from the vector instructions
+        // that made its operands.
         asm volatile(
             "s_nop 1\n\t"
             "v_mfma_f32_4x4x1_16b_f32 %0, %3, %5, %0 cbsz:4 abid:%8\n\t"
@@ -261,24 +264,22 @@ struct MatrixSteps {
             : "+v"(d0), "+v"(d1), "=&v"(e2)
             : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "v"(ea[(K + 2) / NB]), "v"(eb[(K + 2) % NB]), "n"(K % 16), "v"(e1));
       } else {
-        // The leading s_nop separates the first matrix instruction from a register copy the compiler might place
-        // between two statements (it cannot know that the statement opens with a matrix instruction).
+        // No operand of this statement was written by the statement before it (the product comes from two
+        // statements back), so the compiler has no reason to put wait states in between.
         asm volatile(
-            "s_nop 0\n\t"
             "v_mfma_f32_4x4x1_16b_f32 %0, %3, %5, %0 cbsz:4 abid:%8\n\t"
             "v_mul_f32 %2, %6, %7\n\t"
             "v_mfma_f32_4x4x1_16b_f32 %1, %4, %5, %1 cbsz:4 abid:%8"
             : "+v"(d0), "+v"(d1), "=&v"(e2)
-            : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "v"(ea[(K + 2) / NB]), "v"(eb[(K + 2) % NB]), "n"(K % 16), "v"(e1));
+            : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "v"(ea[(K + 2) / NB]), "v"(eb[(K + 2) % NB]), "n"(K % 16));
       }
       MatrixSteps<K + 1, KEND, NB>::run(ea, eb, A, d0, d1, e1, e2);
     } else {
       asm volatile(
-          "s_nop 0\n\t"
           "v_mfma_f32_4x4x1_16b_f32 %0, %2, %4, %0 cbsz:4 abid:%5\n\t"
           "v_mfma_f32_4x4x1_16b_f32 %1, %3, %4, %1 cbsz:4 abid:%5"
           : "+v"(d0), "+v"(d1)
-          : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "n"(K % 16), "v"(e1));
+          : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "n"(K % 16));
       if constexpr (K + 1 < KEND) MatrixSteps<K + 1, KEND, NB>::run(ea, eb, A, d0, d1, e1, e1);
     }
   }
