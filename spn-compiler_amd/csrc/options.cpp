@@ -126,7 +126,7 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       if (o.blocksPerCU < -1 || o.blocksPerCU > 64) throw std::runtime_error("hip-blocks-per-cu must be in [-1,64]");
     } else if (key == "hip-block-size") {
       o.blockSize = parseInt(key, val);
-      if (o.blockSize != 64 && o.blockSize != 128 && o.blockSize != 256 && o.blockSize != 512)
+      if (o.blockSize != 0 && o.blockSize != 64 && o.blockSize != 128 && o.blockSize != 256 && o.blockSize != 512)
         throw std::runtime_error("hip-block-size must be 64, 128, 256 or 512");
     } else if (ignoredKeys().count(key)) {
       // accepted for compatibility, no effect on the HIP target

@@ -30,7 +30,7 @@ struct CompileOptions {
   bool log2Domain = true;                      // "hip-log2-domain": carry log2 values in f32 kernels
   int samplesPerLane = 0;                      // "hip-samples-per-lane": 0 = choose from SPN size
   int jitMaxOps = 20000;                       // "hip-jit-max-ops": above this, auto picks the interpreter
-  int blockSize = 256;                         // "hip-block-size"
+  int blockSize = 0;                           // "hip-block-size": 64, 128, 256 or 512 threads (0 = automatic)
   bool nontemporalLoads = true;                // "hip-nontemporal-loads": mark input loads as streaming
   bool eagerIndices = true;                    // "hip-eager-indices": compute table indices of all features first
   bool jointTables = true;                     // "hip-joint-tables": pair table leaves of a product into joint tables
