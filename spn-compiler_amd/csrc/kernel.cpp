@@ -144,7 +144,12 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
   // when it uses the hardware exp2/log2 instructions.
   const bool hardwareTranscendentals = o.useLogSpace && o.computeType == ComputeType::F32 && o.log2Domain;
   const uint64_t ops = g.nodes.size() + g.stats.productAdds + g.stats.sumTerms * (hardwareTranscendentals ? 1 : 6);
-  bool useInterp = o.kernelMode == KernelMode::Interpreter || (o.kernelMode == KernelMode::Auto && ops > uint64_t(std::max(0, o.jitMaxOps)));
+  // The reference's "maxTaskSize" bounds the operations per compiled task by cutting the graph into several tasks
+  // (mlir/lib/Dialect/LoSPN/Passes/LoSPNTaskPartitioner.cpp:36-148). Here a graph above that bound is not cut:
+  // it goes to the interpreter, whose code size does not depend on the graph.
+  uint64_t jitLimit = uint64_t(std::max(0, o.jitMaxOps));
+  if (o.maxTaskSize > 0) jitLimit = std::min<uint64_t>(jitLimit, uint64_t(o.maxTaskSize));
+  bool useInterp = o.kernelMode == KernelMode::Interpreter || (o.kernelMode == KernelMode::Auto && ops > jitLimit);
   if (useInterp && !o.useLogSpace) {
     if (o.kernelMode == KernelMode::Interpreter) fatal("COMPILATION ERROR: the interpreter kernel supports log-space computation only");
     useInterp = false;

@@ -99,6 +99,13 @@ def test_option_handling(native):
     os.remove(k.fileName())
     with pytest.raises(RuntimeError, match="Could not parse option value"):
         compile_query(native, path, **{"hip-kernel": "magic"})
+    # maxTaskSize: a graph above the bound runs on the interpreter instead of being cut into tasks
+    k = compile_query(native, path, maxTaskSize=10)
+    assert k.info()["kernel_kind"] == 2
+    os.remove(k.fileName())
+    k = compile_query(native, path, maxTaskSize=100000)
+    assert k.info()["kernel_kind"] == 1
+    os.remove(k.fileName())
     with pytest.raises(RuntimeError, match="hip-interp-staged-features must be lds, spill or auto"):
         compile_query(native, path, **{"hip-kernel": "interpreter", "hip-interp-staged-features": "hbm"})
     with pytest.raises(RuntimeError, match="hip-joint-max-entries must be in"):
