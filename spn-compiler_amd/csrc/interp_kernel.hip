@@ -285,6 +285,60 @@ struct MatrixSteps {
   }
 };
 
+// Reads / writes the N slots of a list whose slot numbers sit at head positions pos .. pos+N-1. tier: 0 all in
+// LDS, 1 all in the spill tier, 2 either (select-the-base access). run: the slots are consecutive, so only the
+// first number is read from the head and the others are constant offsets from its address.
+template <int N, bool SPILL>
+__device__ __forceinline__ void readList(const Slots<float, SPILL>& S, const Head& h, int pos, uint32_t tier, bool run, float* out) {
+  if (run) {
+    const uint32_t first = h.word(pos);
+    if (!SPILL || tier == 0) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) out[j] = S.rdLds(first + j);
+    } else if (tier == 1) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) out[j] = S.rdSpill(first + j);
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) out[j] = S.rd(first + j);
+    }
+  } else if (!SPILL || tier == 0) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) out[j] = S.rdLds(h.word(pos + j));
+  } else if (tier == 1) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) out[j] = S.rdSpill(h.word(pos + j));
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) out[j] = S.rd(h.word(pos + j));
+  }
+}
+template <int N, bool SPILL>
+__device__ __forceinline__ void writeList(const Slots<float, SPILL>& S, const Head& h, int pos, uint32_t tier, bool run, const float* v) {
+  if (run) {
+    const uint32_t first = h.word(pos);
+    if (!SPILL || tier == 0) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) S.wrLds(first + j, v[j]);
+    } else if (tier == 1) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) S.wrSpill(first + j, v[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) S.wr(first + j, v[j]);
+    }
+  } else if (!SPILL || tier == 0) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) S.wrLds(h.word(pos + j), v[j]);
+  } else if (tier == 1) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) S.wrSpill(h.word(pos + j), v[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) S.wr(h.word(pos + j), v[j]);
+  }
+}
+
 template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB>
 __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
   typedef Math<float, LOG2> Mt;
@@ -299,33 +353,16 @@ __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, c
     A[g][0] = wl[g * 128];
     A[g][1] = wl[g * 128 + 64];
   }
-  const uint32_t w0 = h.word(1);
-  const bool aScaled = (w0 >> 30) & 1u, bScaled = (w0 >> 31) & 1u, outScaled = (h.word(2) >> 8) & 1u;
+  const uint32_t w0 = h.word(1), w1 = h.word(2);
+  const bool aScaled = (w0 >> 30) & 1u, bScaled = (w0 >> 31) & 1u, outScaled = (w1 >> 8) & 1u;
   float ea[NA], eb[NB];
   // Flagged instructions: the tier bits say per slot list where it lives (valid when exactly the short pool is
   // in LDS), so a list is read with LDS instructions or with scalar-base global loads; mixed lists and other
-  // LDS splits take the select-the-base form.
+  // LDS splits take the select-the-base form. A list that is a run of consecutive slots (bits 9-11 of the second
+  // word) is addressed from its first slot with constant offsets: one lane read and one address for the list.
   const uint32_t tierA = TIERED ? (w0 >> 24) & 3u : 2u, tierB = TIERED ? (w0 >> 26) & 3u : 2u, tierD = TIERED ? (w0 >> 28) & 3u : 2u;
-  if (!SPILL || tierA == 0) {
-#pragma unroll
-    for (int r = 0; r < NA; ++r) ea[r] = S.rdLds(h.word(AS + r));
-  } else if (tierA == 1) {
-#pragma unroll
-    for (int r = 0; r < NA; ++r) ea[r] = S.rdSpill(h.word(AS + r));
-  } else {
-#pragma unroll
-    for (int r = 0; r < NA; ++r) ea[r] = S.rd(h.word(AS + r));
-  }
-  if (!SPILL || tierB == 0) {
-#pragma unroll
-    for (int c = 0; c < NB; ++c) eb[c] = S.rdLds(h.word(BS + c));
-  } else if (tierB == 1) {
-#pragma unroll
-    for (int c = 0; c < NB; ++c) eb[c] = S.rdSpill(h.word(BS + c));
-  } else {
-#pragma unroll
-    for (int c = 0; c < NB; ++c) eb[c] = S.rd(h.word(BS + c));
-  }
+  readList<NA>(S, h, AS, tierA, (w1 >> 9) & 1u, ea);
+  readList<NB>(S, h, BS, tierB, (w1 >> 10) & 1u, eb);
   // A scaled list already holds exp2(value - max) and brings max along in its scale slot; a list of log2
   // values is shifted by its maximum and exponentiated here. All slots are read before any is written.
   float base = 0.f;
@@ -372,16 +409,7 @@ __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, c
       res[4 + t] = base + Mt::log(d1[t]);
     }
   }
-  if (!SPILL || tierD == 0) {
-#pragma unroll
-    for (int t = 0; t < M; ++t) S.wrLds(h.word(DST + t), res[t]);
-  } else if (tierD == 1) {
-#pragma unroll
-    for (int t = 0; t < M; ++t) S.wrSpill(h.word(DST + t), res[t]);
-  } else {
-#pragma unroll
-    for (int t = 0; t < M; ++t) S.wr(h.word(DST + t), res[t]);
-  }
+  writeList<M>(S, h, DST, tierD, (w1 >> 11) & 1u, res);
   return ip + 2 + M + NA + NB + 3 + K * M;
 }
 
@@ -451,6 +479,71 @@ __device__ __forceinline__ code_ptr prodBatch(code_ptr ip, int n, const Slots<R,
   return ip;
 }
 
+// The same for staged features when the program's short pool is exactly what lives in LDS: the second word
+// says in which tier the feature slots (FT) and the destinations (DT) live, 0 LDS or 1 spill tier, so every
+// access is an LDS instruction or a global access from a scalar base instead of a selected generic address.
+// GROUPED: the j-th leaves of the four records of a group read the same feature, which is then read once.
+template <typename R, int G, bool MARGINAL, int FT, int DT, bool GROUPED>
+__device__ __forceinline__ code_ptr prodBatchTiered(code_ptr ip, int n, const Slots<R, true>& S, const InterpLaunch& a) {
+  constexpr int RW = sizeof(R) / 4, LEAF = 1 + 3 * RW, REC = 1 + G * LEAF, P = 4;
+  ip += 2;
+  int done = 0;
+  for (; done + P <= n; done += P, ip += P * REC) {
+    R x[P][G];
+#pragma unroll
+    for (int q = 0; q < (GROUPED ? 1 : P); ++q)
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const uint32_t fw = ip[q * REC + 1 + j * LEAF];
+        x[q][j] = FT == 0 ? S.rdLds(fw) : S.rdSpill(fw);
+      }
+#pragma unroll
+    for (int q = 0; q < P; ++q) {
+      R acc = R(0);
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const long at = q * REC + 1 + j * LEAF + 1;
+        const R xv = x[GROUPED ? 0 : q][j];
+        const R d = xv - constAt<R>(ip, at);
+        R v = rfma(d, d, constAt<R>(ip, at + RW)) * constAt<R>(ip, at + 2 * RW);
+        if (MARGINAL) v = (xv != xv) ? R(0) : v;
+        acc += v;
+      }
+      if (DT == 0) S.wrLds(ip[q * REC], acc);
+      else S.wrSpill(ip[q * REC], acc);
+    }
+  }
+  for (; done < n; ++done, ip += REC) {
+    R acc = R(0);
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+      const uint32_t fw = ip[1 + j * LEAF];
+      const R xv = FT == 0 ? S.rdLds(fw) : S.rdSpill(fw);
+      const R d = xv - constAt<R>(ip, 2 + j * LEAF);
+      R v = rfma(d, d, constAt<R>(ip, 2 + j * LEAF + RW)) * constAt<R>(ip, 2 + j * LEAF + 2 * RW);
+      if (MARGINAL) v = (xv != xv) ? R(0) : v;
+      acc += v;
+    }
+    if (DT == 0) S.wrLds(ip[0], acc);
+    else S.wrSpill(ip[0], acc);
+  }
+  return ip;
+}
+template <typename R, int G, bool MARGINAL, int FT, int DT>
+__device__ __forceinline__ code_ptr prodBatchTieredG(code_ptr ip, int n, bool grouped, const Slots<R, true>& S, const InterpLaunch& a) {
+  if (grouped) return prodBatchTiered<R, G, MARGINAL, FT, DT, true>(ip, n, S, a);
+  return prodBatchTiered<R, G, MARGINAL, FT, DT, false>(ip, n, S, a);
+}
+template <typename R, int G, bool MARGINAL>
+__device__ __forceinline__ code_ptr prodBatchTieredAny(code_ptr ip, int n, uint32_t flags, const Slots<R, true>& S, const InterpLaunch& a) {
+  const uint32_t ft = (flags >> 8) & 3u, dt = (flags >> 10) & 3u;
+  const bool grouped = (flags >> 12) & 1u;
+  if (ft == 0 && dt == 0) return prodBatchTieredG<R, G, MARGINAL, 0, 0>(ip, n, grouped, S, a);
+  if (ft == 0) return prodBatchTieredG<R, G, MARGINAL, 0, 1>(ip, n, grouped, S, a);
+  if (dt == 0) return prodBatchTieredG<R, G, MARGINAL, 1, 0>(ip, n, grouped, S, a);
+  return prodBatchTieredG<R, G, MARGINAL, 1, 1>(ip, n, grouped, S, a);
+}
+
 // Executes one instruction other than OP_END and returns the pointer to the next one.
 template <typename R, bool LOG2, bool SPILL, bool TIERED>
 __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Slots<R, SPILL>& S, const InterpLaunch& a,
@@ -489,7 +582,20 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
   }
   if (op == OP_PRODBATCH) {
     const int n = int(w0 >> 8);
-    const uint32_t leaves = h.word(2);
+    const uint32_t flags = h.word(2), leaves = flags & 0xffu;
+    if constexpr (SPILL && TIERED) {
+      // Tier flags are valid (exactly the short pool is in LDS): no generic accesses unless a list is mixed.
+      if (stagedMode && ((flags >> 8) & 3u) != 2u && ((flags >> 10) & 3u) != 2u && leaves != 3) {
+        if (!a.marginal) {
+          if (leaves == 2) return prodBatchTieredAny<R, 2, false>(ip, n, flags, S, a);
+          if (leaves == 1) return prodBatchTieredAny<R, 1, false>(ip, n, flags, S, a);
+          return prodBatchTieredAny<R, 4, false>(ip, n, flags, S, a);
+        }
+        if (leaves == 2) return prodBatchTieredAny<R, 2, true>(ip, n, flags, S, a);
+        if (leaves == 1) return prodBatchTieredAny<R, 1, true>(ip, n, flags, S, a);
+        return prodBatchTieredAny<R, 4, true>(ip, n, flags, S, a);
+      }
+    }
     // Staged features make the whole batch straight-line code; the direct form decides the input type per read.
     // Without marginal support (the common staged case) the NaN select is not compiled in at all.
     if (stagedMode && !a.marginal) {

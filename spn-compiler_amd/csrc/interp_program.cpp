@@ -5,6 +5,7 @@
 #include <cstring>
 #include <map>
 #include <queue>
+#include <set>
 #include <sstream>
 #include <stdexcept>
 
@@ -319,20 +320,77 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   for (uint32_t k = 0; k < instrs.size(); ++k)
     for (uint32_t d : instrs[k].defs) firstDef[d] = k;
   std::vector<uint32_t> slotOf(N, NONE);
-  typedef std::priority_queue<uint32_t, std::vector<uint32_t>, std::greater<uint32_t>> MinHeap;
-  MinHeap freeShort, freeLong;
+  // Each pool (short-lived slots, long-lived slots) hands out single slots and, with vector blocks switched on,
+  // blocks of nine consecutive slots: the eight results of a matrix-form outer sum and the scale of a scaled
+  // vector, which the kernel then addresses by the first slot alone. Singles are carved out of blocks; a block
+  // whose nine slots are free again is whole again, so the slots of a batch of products that has died serve
+  // the vector computed from it.
+  constexpr uint32_t VECTOR_BLOCK = 9;
+  const bool useBlocks = o.interpVectorBlocks;
+  struct Pool {
+    uint32_t origin = 0;  // number of the pool's first slot (blocks are aligned to it)
+    std::set<uint32_t> singles, wholeBlocks;
+  };
+  Pool shortPool, longPool;
+  shortPool.origin = nextSlot;
+  longPool.origin = LONG_BIT | longCount;
   uint32_t highWater = nextSlot;
+  auto grow = [&](bool isLong, uint32_t count) {
+    uint32_t first;
+    if (isLong) {
+      first = LONG_BIT | longCount;
+      longCount += count;
+    } else {
+      first = highWater;
+      highWater += count;
+    }
+    return first;
+  };
+  auto takeBlock = [&](bool isLong) {
+    Pool& pool = isLong ? longPool : shortPool;
+    if (!pool.wholeBlocks.empty()) {
+      const uint32_t base = *pool.wholeBlocks.begin();
+      pool.wholeBlocks.erase(pool.wholeBlocks.begin());
+      return base;
+    }
+    return grow(isLong, VECTOR_BLOCK);
+  };
   auto allocSlot = [&](uint32_t node) {
     const bool isLong = lastUse[node] - firstDef[node] > longRange;
-    MinHeap& heap = isLong ? freeLong : freeShort;
-    if (!heap.empty()) {
-      uint32_t s = heap.top();
-      heap.pop();
-      return s;
+    Pool& pool = isLong ? longPool : shortPool;
+    if (pool.singles.empty()) {
+      if (!useBlocks) return grow(isLong, 1);
+      const uint32_t base = takeBlock(isLong);
+      for (uint32_t j = 0; j < VECTOR_BLOCK; ++j) pool.singles.insert(base + j);
     }
-    return isLong ? (LONG_BIT | longCount++) : highWater++;
+    const uint32_t s = *pool.singles.begin();
+    pool.singles.erase(pool.singles.begin());
+    return s;
   };
-  auto releaseSlot = [&](uint32_t s) { ((s & LONG_BIT) ? freeLong : freeShort).push(s); };
+  auto releaseSlot = [&](uint32_t s) {
+    Pool& pool = (s & LONG_BIT) ? longPool : shortPool;
+    pool.singles.insert(s);
+    if (!useBlocks) return;
+    const uint32_t base = pool.origin + (s - pool.origin) / VECTOR_BLOCK * VECTOR_BLOCK;
+    for (uint32_t j = 0; j < VECTOR_BLOCK; ++j)
+      if (!pool.singles.count(base + j)) return;
+    for (uint32_t j = 0; j < VECTOR_BLOCK; ++j) pool.singles.erase(base + j);
+    pool.wholeBlocks.insert(base);
+  };
+  struct Block {
+    uint32_t base, live;
+  };
+  std::vector<Block> blocks;
+  std::vector<int> blockOfNode(N, -1);
+  auto allocBlock = [&](uint32_t node) { return takeBlock(lastUse[node] - firstDef[node] > longRange); };
+  auto releaseNode = [&](uint32_t node) {
+    if (blockOfNode[node] < 0) {
+      releaseSlot(slotOf[node]);
+      return;
+    }
+    Block& blk = blocks[size_t(blockOfNode[node])];
+    if (--blk.live == 0) ((blk.base & LONG_BIT) ? longPool : shortPool).wholeBlocks.insert(blk.base);
+  };
   std::vector<size_t> longWords;  // positions in p.code holding long-pool slot numbers
   auto slotWord = [&](uint32_t s) {
     if (s & LONG_BIT) longWords.push_back(p.code.size());
@@ -386,14 +444,34 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
     } else {
       const size_t at = b.begin();
       b.word(OP_PRODBATCH | batchFlag | (uint32_t(batch.size()) << 8));
-      b.word(uint32_t(batch[0].leaves.size()));
+      // Second word: leaves per product; bits 8-9 / 10-11 the tier of the staged feature slots / of the
+      // destinations (0 all in the short pool, 1 all in the long pool, 2 mixed); bit 12: within every full
+      // group of four records the j-th leaves all read the same feature (the leaf regions of a region graph
+      // are like that), so the kernel reads each feature of a group once.
+      // The records do not depend on each other: those that read the same features are put next to each other.
+      auto features = [&](const BatchEntry& e) {
+        std::vector<uint32_t> f;
+        for (uint32_t c : e.leaves) f.push_back(g.nodes[c].feature);
+        return f;
+      };
+      std::stable_sort(batch.begin(), batch.end(), [&](const BatchEntry& x, const BatchEntry& y) { return features(x) < features(y); });
+      uint32_t longDsts = 0;
+      for (const auto& e : batch) longDsts += (e.dst & LONG_BIT) ? 1 : 0;
+      const uint32_t dstTier = longDsts == 0 ? 0u : (longDsts == batch.size() ? 1u : 2u);
+      const uint32_t featTier = p.featureMode == FEAT_STAGED && stagedLong ? 1u : 0u;
+      bool grouped = batch.size() >= 4;
+      for (size_t q = 0; q + 4 <= batch.size() && grouped; q += 4)
+        for (size_t r = 1; r < 4; ++r)
+          for (size_t j = 0; j < batch[q].leaves.size(); ++j)
+            if (g.nodes[batch[q + r].leaves[j]].feature != g.nodes[batch[q].leaves[j]].feature) grouped = false;
+      b.word(uint32_t(batch[0].leaves.size()) | (featTier << 8) | (dstTier << 10) | (grouped ? 0x1000u : 0u));
       for (const auto& e : batch) {
         slotWord(e.dst);
         for (uint32_t c : e.leaves) emitInlineLeaf(c);
       }
       b.end(at);
       b.txt << "  " << slotName(batch[0].dst) << ".. = prodbatch(" << batch.size() << " products x " << batch[0].leaves.size()
-            << " gaussians)   ; nodes " << batch[0].node << "..\n";
+            << " gaussians)" << (grouped ? " grouped" : "") << "   ; nodes " << batch[0].node << "..\n";
     }
     batch.clear();
   };
@@ -408,11 +486,20 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       uniq.erase(std::unique(uniq.begin(), uniq.end()), uniq.end());
       for (uint32_t s : uniq)
         if (lastUse[s] == k) {
-          releaseSlot(slotOf[s]);
-          if (scaleSlotOfNode[s] != NONE) releaseSlot(scaleSlotOfNode[s]);
+          releaseNode(s);
+          if (scaleSlotOfNode[s] != NONE && blockOfNode[s] < 0) releaseSlot(scaleSlotOfNode[s]);  // else part of the block
         }
     }
-    for (uint32_t d : in.defs) slotOf[d] = allocSlot(d);
+    if (in.op == OP_OUTERSUM && matrixInstr[k] && o.interpVectorBlocks) {
+      const uint32_t base = allocBlock(in.defs[0]);
+      for (uint32_t t = 0; t < in.defs.size(); ++t) {
+        slotOf[in.defs[t]] = base + t;
+        blockOfNode[in.defs[t]] = int(blocks.size());
+      }
+      blocks.push_back(Block{base, uint32_t(in.defs.size())});
+    } else {
+      for (uint32_t d : in.defs) slotOf[d] = allocSlot(d);
+    }
     // Bit 7 of the opcode tells the kernel that this instruction touches the long pool.
     uint32_t longFlag = 0;
     for (uint32_t d : in.defs) longFlag |= (slotOf[d] & LONG_BIT) ? 0x80u : 0u;
@@ -490,7 +577,8 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
         const uint32_t scaleA = matrixForm ? scaleSlotOfNode[outer.a[0]] : NONE, scaleB = matrixForm ? scaleSlotOfNode[outer.b[0]] : NONE;
         uint32_t scaleDst = NONE;
         if (matrixForm && linearConsumer[k] >= 0) {
-          scaleDst = allocSlot(in.defs[0]);  // lives exactly as long as the vector
+          // Lives exactly as long as the vector: the ninth slot of its block, or a slot of its own.
+          scaleDst = blockOfNode[in.defs[0]] >= 0 ? slotOf[in.defs[0]] + 8 : allocSlot(in.defs[0]);
           scaleSlotOfNode[in.defs[0]] = scaleDst;
           if (scaleDst & LONG_BIT) longFlag |= 0x80u;
         }
@@ -500,7 +588,14 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
                                                 (scaleA != NONE ? 1u << 30 : 0u) | (scaleB != NONE ? 1u << 31 : 0u)
                                           : 0u;
         b.word((matrixForm ? OP_OUTERMM : OP_OUTERSUM) | longFlag | (na << 8) | (nb << 16) | tiers);
-        b.word(uint32_t(defs.size()) | (scaleDst != NONE ? 0x100u : 0u));
+        // Bits 9-11 of the second word: the a, b and dst lists are runs of consecutive slots.
+        auto consecutive = [&](const std::vector<uint32_t>& nodes) {
+          for (size_t j = 1; j < nodes.size(); ++j)
+            if (slotOf[nodes[j]] != slotOf[nodes[0]] + j) return false;
+          return true;
+        };
+        const uint32_t runs = matrixForm ? (consecutive(outer.a) ? 0x200u : 0u) | (consecutive(outer.b) ? 0x400u : 0u) | (consecutive(defs) ? 0x800u : 0u) : 0u;
+        b.word(uint32_t(defs.size()) | (scaleDst != NONE ? 0x100u : 0u) | runs);
         for (uint32_t d : defs) slotWord(slotOf[d]);
         for (uint32_t a : outer.a) slotWord(slotOf[a]);
         for (uint32_t c : outer.b) slotWord(slotOf[c]);
@@ -528,7 +623,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
     }
     // A value nobody reads later (cannot happen for reachable nodes, kept for safety).
     for (uint32_t d : in.defs)
-      if (d != g.root() && lastUse[d] <= k) releaseSlot(slotOf[d]);
+      if (d != g.root() && lastUse[d] <= k) releaseNode(d);
   }
   flushBatch();
   {

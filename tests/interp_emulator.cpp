@@ -95,9 +95,25 @@ int main(int argc, char** argv) {
           wr(dst, acc);
           pc = q;
         } else if (op == OP_PRODBATCH) {
-          const uint32_t n = w0 >> 8, G = c.at(pc + 1);
+          const uint32_t n = w0 >> 8, w1 = c.at(pc + 1), G = w1 & 0xff;
           if (n < 2 || G < 1 || G > 4) throw std::runtime_error("malformed product batch at word " + std::to_string(pc));
           size_t q = pc + 2;
+          {  // the flags must describe the records: tiers of feature slots and destinations, same feature per group of four
+            const size_t rec = 1 + 4 * size_t(G);
+            uint32_t longFeat = 0, longDst = 0;
+            bool grouped = n >= 4;
+            for (uint32_t i = 0; i < n; ++i) {
+              longDst += c.at(q + i * rec) >= p.shortSlots ? 1 : 0;
+              for (uint32_t j = 0; j < G; ++j) {
+                longFeat += c.at(q + i * rec + 1 + 4 * j) >= p.shortSlots ? 1 : 0;
+                if (i / 4 * 4 + 4 <= n && c.at(q + i * rec + 1 + 4 * j) != c.at(q + (i / 4 * 4) * rec + 1 + 4 * j)) grouped = false;
+              }
+            }
+            const uint32_t dstTier = longDst == 0 ? 0u : (longDst == n ? 1u : 2u);
+            const uint32_t featTier = p.featureMode != FEAT_STAGED ? 0u : (longFeat == 0 ? 0u : (longFeat == n * G ? 1u : 2u));
+            if (((w1 >> 8) & 3) != featTier || ((w1 >> 10) & 3) != dstTier || (((w1 >> 12) & 1) && !grouped))
+              throw std::runtime_error("product batch flags disagree with its records at word " + std::to_string(pc));
+          }
           for (uint32_t i = 0; i < n; ++i) {
             const uint32_t dst = c.at(q++);
             float acc = 0;
@@ -141,6 +157,16 @@ int main(int argc, char** argv) {
           const uint32_t na = (w0 >> 8) & 0xff, nb = (w0 >> 16) & 0xff, M = c.at(pc + 1) & 0xff;
           const size_t d0 = pc + 2, a0 = d0 + M, b0 = a0 + na, sc = b0 + nb, w = sc + (mm ? 3 : 0);
           const bool aScaled = mm && ((w0 >> 30) & 1), bScaled = mm && ((w0 >> 31) & 1), outScaled = mm && ((c.at(pc + 1) >> 8) & 1);
+          if (mm) {  // a list flagged as a run must consist of consecutive slots (the kernel then reads only its first number)
+            auto isRun = [&](size_t first, uint32_t count) {
+              for (uint32_t j = 1; j < count; ++j)
+                if (c.at(first + j) != c.at(first) + j) return false;
+              return true;
+            };
+            const uint32_t w1 = c.at(pc + 1);
+            if ((((w1 >> 9) & 1) && !isRun(a0, na)) || (((w1 >> 10) & 1) && !isRun(b0, nb)) || (((w1 >> 11) & 1) && !isRun(d0, M)))
+              throw std::runtime_error("run flag on a list of non-consecutive slots at word " + std::to_string(pc));
+          }
           if (mm) {
             if (M != 8 || (na * nb) % 16 != 0) throw std::runtime_error("malformed matrix-form outer sum at word " + std::to_string(pc));
             auto tier = [&](size_t first, uint32_t count) {  // the tier bits must describe the slot lists

@@ -206,12 +206,17 @@ def test_generated_source_variants(native):
     assert i["trans_min"] < i["sum_terms"] // 10 and i["flops_min"] < 2 * i["sum_terms"]
     os.remove(k.fileName())
     # the program builder honours the tier and pool-size options
-    k = compile_spn(native, syn.c4_spn(), "float32", **{"hip-interp-staged-features": "lds", "hip-interp-long-range": 8, "hip-interp-short-slots": 40})
+    pools = {"hip-interp-staged-features": "lds", "hip-interp-long-range": 8, "hip-interp-short-slots": 40}
+    k = compile_spn(native, syn.c4_spn(), "float32", **pools)
+    src = k.source()
+    os.remove(k.fileName())
+    # region vectors take blocks of nine consecutive slots (eight values and the scale): 32 features + one block
+    assert "149 value slots (32 staged features, 108 long-lived)" in src and "prodbatch(8 products x 2 gaussians) grouped" in src
+    k = compile_spn(native, syn.c4_spn(), "float32", **pools, **{"hip-interp-vector-blocks": "false"})
     assert "140 value slots (32 staged features, 99 long-lived)" in k.source()   # 41 = 32 features + one vector of 8 and its scale
     assert k.source().count(") scaled ") == 140             # every region vector that only feeds another region
     os.remove(k.fileName())
-    k = compile_spn(native, syn.c4_spn(), "float32", **{"hip-interp-scaled-vectors": "false", "hip-interp-staged-features": "lds",
-                                                        "hip-interp-long-range": 8, "hip-interp-short-slots": 40})
+    k = compile_spn(native, syn.c4_spn(), "float32", **pools, **{"hip-interp-scaled-vectors": "false", "hip-interp-vector-blocks": "false"})
     assert "136 value slots (32 staged features, 96 long-lived)" in k.source() and ") scaled " not in k.source()
     os.remove(k.fileName())
 
