@@ -339,6 +339,39 @@ __device__ __forceinline__ void writeList(const Slots<float, SPILL>& S, const He
   }
 }
 
+// The matrix chain over the products ea[r] * eb[c] and what follows it: results as log2 values (base + log2 of
+// each sum), or as a scaled vector, acc_t / max(acc) with base + log2(max) in the scale slot. dstPos / scalePos
+// are the head positions of the eight destinations and of the scale slot.
+template <bool LOG2, bool SPILL, int NA, int NB>
+__device__ __forceinline__ void matrixChainAndStore(const float* ea, const float* eb, const float (*A)[2], float base, bool outScaled,
+                                                    const Head& h, int dstPos, int scalePos, uint32_t tierD, bool dstRun,
+                                                    const Slots<float, SPILL>& S) {
+  typedef Math<float, LOG2> Mt;
+  constexpr int M = 8, K = NA * NB;
+  float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+  MatrixSteps<0, K, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
+  float res[M];
+  if (outScaled) {
+    // acc_t / max(acc) and one logarithm for the whole vector. All-zero accumulators (impossible evidence) give
+    // zeros and a scale of -inf; the floor under the maximum only keeps the reciprocal finite.
+    float m = rmax(rmax(rmax(d0[0], d0[1]), rmax(d0[2], d0[3])), rmax(rmax(d1[0], d1[1]), rmax(d1[2], d1[3])));
+    const float inv = __builtin_amdgcn_rcpf(rmax(m, 0x1p-100f));
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      res[t] = d0[t] * inv;
+      res[4 + t] = d1[t] * inv;
+    }
+    S.wr(h.word(scalePos), base + Mt::log(m));
+  } else {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      res[t] = base + Mt::log(d0[t]);
+      res[4 + t] = base + Mt::log(d1[t]);
+    }
+  }
+  writeList<M>(S, h, dstPos, tierD, dstRun, res);
+}
+
 template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB>
 __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
   typedef Math<float, LOG2> Mt;
@@ -388,28 +421,7 @@ __device__ __forceinline__ code_ptr outerSumMatrix(code_ptr ip, const Head& h, c
     for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(eb[c] - mb);
     base += mb;
   }
-  float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
-  MatrixSteps<0, K, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
-  float res[M];
-  if (outScaled) {
-    // acc_t / max(acc) and one logarithm for the whole vector. All-zero accumulators (impossible evidence) give
-    // zeros and a scale of -inf; the floor under the maximum only keeps the reciprocal finite.
-    float m = rmax(rmax(rmax(d0[0], d0[1]), rmax(d0[2], d0[3])), rmax(rmax(d1[0], d1[1]), rmax(d1[2], d1[3])));
-    const float inv = __builtin_amdgcn_rcpf(rmax(m, 0x1p-100f));
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      res[t] = d0[t] * inv;
-      res[4 + t] = d1[t] * inv;
-    }
-    S.wr(h.word(SCALES), base + Mt::log(m));
-  } else {
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      res[t] = base + Mt::log(d0[t]);
-      res[4 + t] = base + Mt::log(d1[t]);
-    }
-  }
-  writeList<M>(S, h, DST, tierD, (w1 >> 11) & 1u, res);
+  matrixChainAndStore<LOG2, SPILL, NA, NB>(ea, eb, A, base, outScaled, h, DST, SCALES, tierD, (w1 >> 11) & 1u, S);
   return ip + 2 + M + NA + NB + 3 + K * M;
 }
 
@@ -430,6 +442,77 @@ __device__ __forceinline__ code_ptr outerSumNB(code_ptr ip, int na, int nb, cons
   if (nb == 4) return outerSum<R, LOG2, SPILL, M, 4>(ip, na, S);
   if (nb == 16) return outerSum<R, LOG2, SPILL, M, 16>(ip, na, S);
   return outerSum<R, LOG2, SPILL, M, 2>(ip, na, S);
+}
+
+// OP_LEAFMM: the operand lists are products of G Gaussian leaves, all products of a list over the same G features.
+// Weights, features and leaf constants are requested together; the products stay in registers.
+template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB, int G, bool MARGINAL>
+__device__ __forceinline__ code_ptr leafRegionMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
+  typedef Math<float, LOG2> Mt;
+  constexpr int M = 8, K = NA * NB, GROUPS = K / 16;
+  // Head: length, opcode, format, eight destinations, the scale slot, 2 G feature slots. ip points at the opcode.
+  constexpr int DST = 3, SCALE = DST + M, FEAT = SCALE + 1, REC = FEAT + 2 * G - 1;  // REC: offset of the constants from ip
+  float A[GROUPS][2];
+  const float* wl = wGlobal + (threadIdx.x & 63u);
+#pragma unroll
+  for (int g = 0; g < GROUPS; ++g) {
+    A[g][0] = wl[g * 128];
+    A[g][1] = wl[g * 128 + 64];
+  }
+  const uint32_t w0 = h.word(1), w1 = h.word(2);
+  const uint32_t tierD = TIERED ? (w0 >> 28) & 3u : 2u, tierF = TIERED ? (w1 >> 16) & 3u : 2u;
+  float x[2 * G];
+  if (!SPILL || tierF == 0) {
+#pragma unroll
+    for (int j = 0; j < 2 * G; ++j) x[j] = S.rdLds(h.word(FEAT + j));
+  } else if (tierF == 1) {
+#pragma unroll
+    for (int j = 0; j < 2 * G; ++j) x[j] = S.rdSpill(h.word(FEAT + j));
+  } else {
+#pragma unroll
+    for (int j = 0; j < 2 * G; ++j) x[j] = S.rd(h.word(FEAT + j));
+  }
+  float e[NA + NB];
+#pragma unroll
+  for (int i = 0; i < NA + NB; ++i) {
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+      const long at = REC + (i * G + j) * 3;
+      const float xv = x[(i < NA ? 0 : G) + j];
+      const float d = xv - constAt<float>(ip, at);
+      float v = rfma(d, d, constAt<float>(ip, at + 1)) * constAt<float>(ip, at + 2);
+      if (MARGINAL) v = (xv != xv) ? 0.f : v;
+      acc += v;
+    }
+    e[i] = acc;
+  }
+  float ma = -__builtin_huge_valf(), mb = -__builtin_huge_valf();
+#pragma unroll
+  for (int r = 0; r < NA; ++r) ma = rmax(ma, e[r]);
+#pragma unroll
+  for (int c = 0; c < NB; ++c) mb = rmax(mb, e[NA + c]);
+  ma = rmax(ma, Mt::lowest());
+  mb = rmax(mb, Mt::lowest());
+  float ea[NA], eb[NB];
+#pragma unroll
+  for (int r = 0; r < NA; ++r) ea[r] = Mt::exp(e[r] - ma);
+#pragma unroll
+  for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(e[NA + c] - mb);
+  matrixChainAndStore<LOG2, SPILL, NA, NB>(ea, eb, A, ma + mb, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
+  return ip + 2 + M + 1 + 2 * G + (NA + NB) * G * 3 + K * M;
+}
+template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB>
+__device__ __forceinline__ code_ptr leafRegionMatrixG(code_ptr ip, const Head& h, uint32_t leaves, bool marginal, const float* wGlobal,
+                                                       const Slots<float, SPILL>& S) {
+  if (!marginal) {
+    if (leaves == 2) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 2, false>(ip, h, wGlobal, S);
+    if (leaves == 1) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 1, false>(ip, h, wGlobal, S);
+    return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 4, false>(ip, h, wGlobal, S);
+  }
+  if (leaves == 2) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 2, true>(ip, h, wGlobal, S);
+  if (leaves == 1) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 1, true>(ip, h, wGlobal, S);
+  return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 4, true>(ip, h, wGlobal, S);
 }
 
 // n products of G Gaussian leaves each. The records are independent, so they are taken four at
@@ -642,6 +725,13 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
   }
   const int na = int((w0 >> 8) & 0xffu), nb = int((w0 >> 16) & 0xffu);
   if constexpr (sizeof(R) == 4) {
+    if (op == OP_LEAFMM) {
+      // The weights start after the two header words, eight destinations, the scale slot, the feature slots and the leaf constants.
+      const uint32_t leaves = (h.word(2) >> 12) & 0xfu;
+      const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 11 + 2 * leaves + (na + nb) * leaves * 3);
+      if (na == 4) return leafRegionMatrixG<LOG2, SPILL, TIERED, 4, 4>(ip, h, leaves, a.marginal != 0, wGlobal, S);
+      return leafRegionMatrixG<LOG2, SPILL, TIERED, 8, 8>(ip, h, leaves, a.marginal != 0, wGlobal, S);
+    }
     if (op == OP_OUTERMM) {
       // The weights start after the two header words, eight destinations, na + nb operands and three scale slots.
       const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 13 + na + nb);

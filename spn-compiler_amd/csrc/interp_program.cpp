@@ -282,6 +282,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   // exponential for that list and the producer one logarithm instead of eight.
   std::vector<bool> matrixInstr(instrs.size(), false);
   std::vector<int> linearConsumer(instrs.size(), -1);  // producer -> consuming instruction
+  std::vector<bool> leafRegion(instrs.size(), false), fusedProduct(instrs.size(), false);
   {
     for (uint32_t k = 0; k < instrs.size(); ++k) {
       const Instr& in = instrs[k];
@@ -307,6 +308,40 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       if (!ok || consumer < 0 || !matrixInstr[consumer]) continue;
       const Outer& co = outerOf.at(g.nodes[instrs[consumer].node].children);
       if (co.a == in.defs || co.b == in.defs) linearConsumer[k] = consumer;
+    }
+    // Leaf regions: a matrix-form outer sum over two lists of products of Gaussian leaves only, each product
+    // read by nothing else and all products of a list over the same features, computes them itself. The
+    // product instructions disappear and with them their slots.
+    std::vector<uint32_t> instrOfNode(N, NONE);
+    for (uint32_t k = 0; k < instrs.size(); ++k)
+      for (uint32_t d : instrs[k].defs) instrOfNode[d] = k;
+    auto leafFeatures = [&](uint32_t node, std::vector<uint32_t>& out) {
+      const auto& pn = g.nodes[node];
+      if (pn.kind != NodeKind::Product || node == g.root() || readers[node].size() != 1) return false;
+      for (uint32_t c : pn.children) {
+        if (!inlined[c] || g.nodes[c].kind != NodeKind::Gaussian) return false;
+        out.push_back(g.nodes[c].feature);
+      }
+      return true;
+    };
+    for (uint32_t k = 0; k < instrs.size() && o.interpLeafRegions && p.featureMode == FEAT_STAGED; ++k) {
+      if (!matrixInstr[k]) continue;
+      const Outer& outer = outerOf.at(g.nodes[instrs[k].node].children);
+      if (!((outer.a.size() == 4 && outer.b.size() == 4) || (outer.a.size() == 8 && outer.b.size() == 8))) continue;
+      bool ok = true;
+      std::vector<uint32_t> fa, fb;
+      for (const std::vector<uint32_t>* list : {&outer.a, &outer.b}) {
+        std::vector<uint32_t>& want = list == &outer.a ? fa : fb;
+        for (size_t r = 0; r < list->size() && ok; ++r) {
+          std::vector<uint32_t> f;
+          ok = leafFeatures((*list)[r], f) && (r == 0 || f == want);
+          if (r == 0) want = f;
+        }
+      }
+      if (!ok || fa.size() != fb.size() || !(fa.size() == 1 || fa.size() == 2 || fa.size() == 4)) continue;
+      leafRegion[k] = true;
+      for (uint32_t s : instrs[k].srcs) fusedProduct[instrOfNode[s]] = true;
+      instrs[k].srcs.clear();
     }
   }
   std::vector<uint32_t> scaleSlotOfNode(N, NONE);  // first result of a scaled linear vector -> slot of its scale
@@ -478,6 +513,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
 
   for (uint32_t k = 0; k < instrs.size(); ++k) {
     const Instr& in = instrs[k];
+    if (fusedProduct[k]) continue;  // computed inside the outer sum that reads it
     // Sources dying here release their slots before the destinations are chosen: every
     // opcode reads all of its operands before it writes.
     {
@@ -584,16 +620,43 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
         }
         if (scaleA != NONE && (scaleA & LONG_BIT)) longFlag |= 0x80u;
         if (scaleB != NONE && (scaleB & LONG_BIT)) longFlag |= 0x80u;
-        const uint32_t tiers = matrixForm ? (tierOf(outer.a) << 24) | (tierOf(outer.b) << 26) | (tierOf(defs) << 28) |
-                                                (scaleA != NONE ? 1u << 30 : 0u) | (scaleB != NONE ? 1u << 31 : 0u)
-                                          : 0u;
-        b.word((matrixForm ? OP_OUTERMM : OP_OUTERSUM) | longFlag | (na << 8) | (nb << 16) | tiers);
-        // Bits 9-11 of the second word: the a, b and dst lists are runs of consecutive slots.
         auto consecutive = [&](const std::vector<uint32_t>& nodes) {
           for (size_t j = 1; j < nodes.size(); ++j)
             if (slotOf[nodes[j]] != slotOf[nodes[0]] + j) return false;
           return true;
         };
+        if (leafRegion[k]) {
+          const uint32_t G = uint32_t(g.nodes[outer.a[0]].children.size());
+          if (stagedLong) longFlag |= 0x80u;
+          b.word(OP_LEAFMM | longFlag | (na << 8) | (nb << 16) | (tierOf(defs) << 28));
+          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | (stagedLong ? 1u << 16 : 0u));
+          for (uint32_t d : defs) slotWord(slotOf[d]);
+          if (scaleDst != NONE) slotWord(scaleDst);
+          else b.word(NONE);
+          for (uint32_t list : {outer.a[0], outer.b[0]})
+            for (uint32_t c : g.nodes[list].children) slotWord(valueSlotOf[g.nodes[c].feature]);
+          for (const std::vector<uint32_t>* list : {&outer.a, &outer.b})
+            for (uint32_t prod : *list)
+              for (uint32_t c : g.nodes[prod].children) {
+                const auto& leaf = g.nodes[c];
+                const double coef = -std::log(leaf.stddev) + -0.5 * std::log(2 * M_PI), den = -(1.0 / (2.0 * leaf.stddev * leaf.stddev));
+                b.real(leaf.mean);
+                b.real(coef / den);
+                b.real(den * b.scale);
+              }
+          for (uint32_t grp = 0; grp < na * nb / 16; ++grp)
+            for (uint32_t half = 0; half < 2; ++half)
+              for (uint32_t lane = 0; lane < 64; ++lane) b.real(g.nodes[defs[half * 4 + lane % 4]].weights[grp * 16 + lane / 4]);
+          b.end(at);
+          b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = leafregion(8 sums x " << na << "x" << nb << " products of " << G << " gaussians)"
+                << (scaleDst != NONE ? " scaled" : "") << "   ; nodes " << in.defs[0] << "..\n";
+          break;
+        }
+        const uint32_t tiers = matrixForm ? (tierOf(outer.a) << 24) | (tierOf(outer.b) << 26) | (tierOf(defs) << 28) |
+                                                (scaleA != NONE ? 1u << 30 : 0u) | (scaleB != NONE ? 1u << 31 : 0u)
+                                          : 0u;
+        b.word((matrixForm ? OP_OUTERMM : OP_OUTERSUM) | longFlag | (na << 8) | (nb << 16) | tiers);
+        // Bits 9-11 of the second word: the a, b and dst lists are runs of consecutive slots.
         const uint32_t runs = matrixForm ? (consecutive(outer.a) ? 0x200u : 0u) | (consecutive(outer.b) ? 0x400u : 0u) | (consecutive(defs) ? 0x800u : 0u) : 0u;
         b.word(uint32_t(defs.size()) | (scaleDst != NONE ? 0x100u : 0u) | runs);
         for (uint32_t d : defs) slotWord(slotOf[d]);

@@ -34,6 +34,10 @@ enum InterpOp : uint32_t {
                     //   OUTERSUM for float, eight sums and NA*NB a multiple of 16: weight of product k = r*NB + c and
                     //   sum t sits at word (k/16)*128 + (t/4)*64 + (k%16)*4 + t%4, i.e. 64-word rows that one
                     //   wavefront loads with one coalesced access and that feed sixteen 4x4x1 matrix instructions
+  OP_LEAFMM = 7,    // [op|NA<<8|NB<<16|dstTier<<28][8|outScaled<<8|dstRun<<11|G<<12|featTier<<16] dst*8, scaleDst (or
+                    //   0xFFFFFFFF), G feature slots of the a list, G of the b list, (NA+NB)*G*(mean, shift, den),
+                    //   weights as in OP_OUTERMM: an OP_OUTERMM whose operand lists are products of G Gaussian leaves
+                    //   each, all products of a list over the same features; they are computed in registers
   OP_PRODBATCH = 5, // [op|n<<8][G|featTier<<8|dstTier<<10|grouped<<12] n*(dst, G*(feat, mean, shift, den))
                     //   n products of G Gaussian leaves each; the records are independent of each other.
                     //   Tiers as in OP_OUTERMM (0 short pool, 1 long pool, 2 mixed); grouped: in every full group

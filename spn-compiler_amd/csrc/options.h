@@ -39,6 +39,7 @@ struct CompileOptions {
   int tableBudgetKiB = 62;                     // "hip-table-budget-kib": LDS the table pool may grow to when leaves are paired into joint tables
   int jointMaxEntries = 160;                   // "hip-joint-max-entries": largest joint table (entries) a pair of table leaves may get
   int interpShortSlots = 0;                    // "hip-interp-short-slots": LDS value slots per lane the interpreter program aims for (0 = automatic)
+  bool interpLeafRegions = true;               // "hip-interp-leaf-regions": Gaussian leaf products read by one matrix-form outer sum are computed inside it
   bool interpVectorBlocks = true;              // "hip-interp-vector-blocks": results of a matrix-form outer sum occupy consecutive slots
   bool interpScaledVectors = true;             // "hip-interp-scaled-vectors": region vectors between matrix-form outer sums travel as scaled linear values
   bool interpMatrixCore = true;                // "hip-interp-matrix-core": float outer sums of eight sums run on the matrix cores

@@ -215,6 +215,58 @@ int main(int argc, char** argv) {
             for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), base + lg(res[t]));
           }
           pc = w + size_t(na) * nb * M;
+        } else if (op == OP_LEAFMM) {
+          // An outer sum in matrix form whose operands are products of G Gaussian leaves, computed on the spot.
+          const uint32_t na = (w0 >> 8) & 0xff, nb = (w0 >> 16) & 0xff, w1 = c.at(pc + 1), M = w1 & 0xff, G = (w1 >> 12) & 0xf;
+          const bool outScaled = (w1 >> 8) & 1;
+          if (M != 8 || !((na == 4 && nb == 4) || (na == 8 && nb == 8)) || !(G == 1 || G == 2 || G == 4) || p.featureMode != FEAT_STAGED)
+            throw std::runtime_error("malformed leaf region at word " + std::to_string(pc));
+          const size_t d0 = pc + 2, sc = d0 + M, f0 = sc + 1, r0 = f0 + 2 * G, w = r0 + size_t(na + nb) * G * 3;
+          uint32_t longDst = 0, longFeat = 0;
+          for (uint32_t t = 0; t < M; ++t) longDst += c.at(d0 + t) >= p.shortSlots ? 1 : 0;
+          for (uint32_t j = 0; j < 2 * G; ++j) longFeat += c.at(f0 + j) >= p.shortSlots ? 1 : 0;
+          if (((w0 >> 28) & 3) != (longDst == 0 ? 0u : (longDst == M ? 1u : 2u)) || (longFeat != 0 && longFeat != 2 * G) ||
+              ((w1 >> 16) & 3) != (longFeat ? 1u : 0u))
+            throw std::runtime_error("tier bits disagree with the slot lists at word " + std::to_string(pc));
+          if ((w1 >> 11) & 1)
+            for (uint32_t t = 1; t < M; ++t)
+              if (c.at(d0 + t) != c.at(d0) + t) throw std::runtime_error("run flag on a list of non-consecutive slots at word " + std::to_string(pc));
+          if ((c.at(sc) != UINT32_MAX) != outScaled) throw std::runtime_error("scale slot disagrees with the format bit at word " + std::to_string(pc));
+          std::vector<float> e(na + nb);
+          for (uint32_t i = 0; i < na + nb; ++i) {
+            float acc = 0;
+            for (uint32_t j = 0; j < G; ++j) {
+              const size_t q = r0 + (size_t(i) * G + j) * 3;
+              const float xv = rd(c.at(f0 + (i < na ? 0 : G) + j));
+              const float d = xv - asFloat(c.at(q));
+              float v = (d * d + asFloat(c.at(q + 1))) * asFloat(c.at(q + 2));
+              if (g.supportMarginal && xv != xv) v = 0;
+              acc += v;
+            }
+            e[i] = acc;
+          }
+          float ma = -INFINITY, mb = -INFINITY;
+          for (uint32_t r = 0; r < na; ++r) ma = std::fmax(ma, e[r]);
+          for (uint32_t cc = 0; cc < nb; ++cc) mb = std::fmax(mb, e[na + cc]);
+          ma = std::fmax(ma, -3.4028234663852886e38f);
+          mb = std::fmax(mb, -3.4028234663852886e38f);
+          std::vector<float> res(M, 0.f);
+          for (uint32_t t = 0; t < M; ++t)
+            for (uint32_t r = 0; r < na; ++r)
+              for (uint32_t cc = 0; cc < nb; ++cc) {
+                const uint32_t k = r * nb + cc;
+                res[t] += ex(e[r] - ma) * ex(e[na + cc] - mb) * asFloat(c.at(w + (k / 16) * 128 + (t / 4) * 64 + (k % 16) * 4 + t % 4));
+              }
+          if (outScaled) {
+            float m = 0.f;
+            for (uint32_t t = 0; t < M; ++t) m = std::fmax(m, res[t]);
+            const float inv = 1.0f / std::fmax(m, 0x1p-100f);
+            for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), res[t] * inv);
+            wr(c.at(sc), ma + mb + lg(m));
+          } else {
+            for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), ma + mb + lg(res[t]));
+          }
+          pc = w + size_t(na) * nb * M;
         } else {
           throw std::runtime_error("unknown opcode at word " + std::to_string(pc));
         }

@@ -199,14 +199,18 @@ def test_generated_source_variants(native):
     k = compile_spn(native, syn.c4_spn(), "float32")
     src = k.source()
     assert k.info()["kernel_kind"] == 2 and "outersum(8 sums x 8x8 products)" in src
-    # leaf products come in batches of eight (two leaf regions of four), 80 leaf regions pairs in all
-    assert src.count("prodbatch(8 products x 2 gaussians)") == 80 and " = prod(" not in src
+    # the 80 pairs of leaf regions are computed inside the outer sums over them: no product instructions at all
+    assert src.count("leafregion(8 sums x 4x4 products of 2 gaussians) scaled") == 80 and " = prod(" not in src and "prodbatch" not in src
+    k2 = compile_spn(native, syn.c4_spn(), "float32", **{"hip-interp-leaf-regions": "false"})
+    # without that, leaf products come in batches of eight (two leaf regions of four), sorted by feature
+    assert k2.source().count("prodbatch(8 products x 2 gaussians) grouped") == 80 and "leafregion" not in k2.source()
+    os.remove(k2.fileName())
     # outer-product sums are priced in their factored form: far fewer exponentials than sum terms
     i = k.info()
     assert i["trans_min"] < i["sum_terms"] // 10 and i["flops_min"] < 2 * i["sum_terms"]
     os.remove(k.fileName())
     # the program builder honours the tier and pool-size options
-    pools = {"hip-interp-staged-features": "lds", "hip-interp-long-range": 8, "hip-interp-short-slots": 40}
+    pools = {"hip-interp-staged-features": "lds", "hip-interp-long-range": 8, "hip-interp-short-slots": 40, "hip-interp-leaf-regions": "false"}
     k = compile_spn(native, syn.c4_spn(), "float32", **pools)
     src = k.source()
     os.remove(k.fileName())
