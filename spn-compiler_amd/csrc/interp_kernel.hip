@@ -444,11 +444,45 @@ __device__ __forceinline__ code_ptr outerSumNB(code_ptr ip, int na, int nb, cons
   return outerSum<R, LOG2, SPILL, M, 2>(ip, na, S);
 }
 
+// The operand vectors of a leaf region: NA + NB products of G Gaussian leaves, the first NA over the features
+// x[0..G), the others over x[G..2G); constants (mean, shift, den per leaf) at ip[rec...]. Returns exp2(product -
+// max) per list in ea / eb and the sum of the two maxima.
+template <bool LOG2, int NA, int NB, int G, bool MARGINAL>
+__device__ __forceinline__ float leafOperands(code_ptr ip, long rec, const float* x, float* ea, float* eb) {
+  typedef Math<float, LOG2> Mt;
+  float e[NA + NB];
+#pragma unroll
+  for (int i = 0; i < NA + NB; ++i) {
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+      const long at = rec + (i * G + j) * 3;
+      const float xv = x[(i < NA ? 0 : G) + j];
+      const float d = xv - constAt<float>(ip, at);
+      float v = rfma(d, d, constAt<float>(ip, at + 1)) * constAt<float>(ip, at + 2);
+      if (MARGINAL) v = (xv != xv) ? 0.f : v;
+      acc += v;
+    }
+    e[i] = acc;
+  }
+  float ma = -__builtin_huge_valf(), mb = -__builtin_huge_valf();
+#pragma unroll
+  for (int r = 0; r < NA; ++r) ma = rmax(ma, e[r]);
+#pragma unroll
+  for (int c = 0; c < NB; ++c) mb = rmax(mb, e[NA + c]);
+  ma = rmax(ma, Mt::lowest());
+  mb = rmax(mb, Mt::lowest());
+#pragma unroll
+  for (int r = 0; r < NA; ++r) ea[r] = Mt::exp(e[r] - ma);
+#pragma unroll
+  for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(e[NA + c] - mb);
+  return ma + mb;
+}
+
 // OP_LEAFMM: the operand lists are products of G Gaussian leaves, all products of a list over the same G features.
 // Weights, features and leaf constants are requested together; the products stay in registers.
 template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB, int G, bool MARGINAL>
 __device__ __forceinline__ code_ptr leafRegionMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
-  typedef Math<float, LOG2> Mt;
   constexpr int M = 8, K = NA * NB, GROUPS = K / 16;
   // Head: length, opcode, format, eight destinations, the scale slot, 2 G feature slots. ip points at the opcode.
   constexpr int DST = 3, SCALE = DST + M, FEAT = SCALE + 1, REC = FEAT + 2 * G - 1;  // REC: offset of the constants from ip
@@ -472,34 +506,9 @@ __device__ __forceinline__ code_ptr leafRegionMatrix(code_ptr ip, const Head& h,
 #pragma unroll
     for (int j = 0; j < 2 * G; ++j) x[j] = S.rd(h.word(FEAT + j));
   }
-  float e[NA + NB];
-#pragma unroll
-  for (int i = 0; i < NA + NB; ++i) {
-    float acc = 0.f;
-#pragma unroll
-    for (int j = 0; j < G; ++j) {
-      const long at = REC + (i * G + j) * 3;
-      const float xv = x[(i < NA ? 0 : G) + j];
-      const float d = xv - constAt<float>(ip, at);
-      float v = rfma(d, d, constAt<float>(ip, at + 1)) * constAt<float>(ip, at + 2);
-      if (MARGINAL) v = (xv != xv) ? 0.f : v;
-      acc += v;
-    }
-    e[i] = acc;
-  }
-  float ma = -__builtin_huge_valf(), mb = -__builtin_huge_valf();
-#pragma unroll
-  for (int r = 0; r < NA; ++r) ma = rmax(ma, e[r]);
-#pragma unroll
-  for (int c = 0; c < NB; ++c) mb = rmax(mb, e[NA + c]);
-  ma = rmax(ma, Mt::lowest());
-  mb = rmax(mb, Mt::lowest());
   float ea[NA], eb[NB];
-#pragma unroll
-  for (int r = 0; r < NA; ++r) ea[r] = Mt::exp(e[r] - ma);
-#pragma unroll
-  for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(e[NA + c] - mb);
-  matrixChainAndStore<LOG2, SPILL, NA, NB>(ea, eb, A, ma + mb, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
+  const float base = leafOperands<LOG2, NA, NB, G, MARGINAL>(ip, REC, x, ea, eb);
+  matrixChainAndStore<LOG2, SPILL, NA, NB>(ea, eb, A, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
   return ip + 2 + M + 1 + 2 * G + (NA + NB) * G * 3 + K * M;
 }
 template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB>
@@ -513,6 +522,78 @@ __device__ __forceinline__ code_ptr leafRegionMatrixG(code_ptr ip, const Head& h
   if (leaves == 2) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 2, true>(ip, h, wGlobal, S);
   if (leaves == 1) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 1, true>(ip, h, wGlobal, S);
   return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 4, true>(ip, h, wGlobal, S);
+}
+
+// OP_LEAFPAIRMM: an 8x8 outer sum whose operand lists are the result vectors of two leaf regions (N x N products
+// of G Gaussian leaves each, eight sums each; N = 4 is what the program builder emits). The two vectors stay in registers as scaled vectors; all weights,
+// features and constants of the three sums are requested at the start.
+template <bool LOG2, bool SPILL, bool TIERED, int N, int G, bool MARGINAL>
+__device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
+  typedef Math<float, LOG2> Mt;
+  constexpr int M = 8, KL = N * N, GL = KL / 16;
+  // Head: length, opcode, format, eight destinations, the scale slot, 4 G feature slots. ip points at the opcode.
+  constexpr int DST = 3, SCALE = DST + M, FEAT = SCALE + 1, REC = FEAT + 4 * G - 1, RECS = 2 * N * G * 3;
+  float A1[GL][2], A2[GL][2], AT[4][2];
+  const float* wl = wGlobal + (threadIdx.x & 63u);
+#pragma unroll
+  for (int g = 0; g < GL; ++g) {
+    A1[g][0] = wl[g * 128];
+    A1[g][1] = wl[g * 128 + 64];
+  }
+#pragma unroll
+  for (int g = 0; g < GL; ++g) {
+    A2[g][0] = wl[KL * M + g * 128];
+    A2[g][1] = wl[KL * M + g * 128 + 64];
+  }
+  const uint32_t w0 = h.word(1), w1 = h.word(2);
+  const uint32_t tierD = TIERED ? (w0 >> 28) & 3u : 2u, tierF = TIERED ? (w1 >> 16) & 3u : 2u;
+  float x[4 * G];
+  if (!SPILL || tierF == 0) {
+#pragma unroll
+    for (int j = 0; j < 4 * G; ++j) x[j] = S.rdLds(h.word(FEAT + j));
+  } else if (tierF == 1) {
+#pragma unroll
+    for (int j = 0; j < 4 * G; ++j) x[j] = S.rdSpill(h.word(FEAT + j));
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4 * G; ++j) x[j] = S.rd(h.word(FEAT + j));
+  }
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    AT[g][0] = wl[2 * KL * M + g * 128];
+    AT[g][1] = wl[2 * KL * M + g * 128 + 64];
+  }
+  float va[M], vb[M], base = 0.f;
+#pragma unroll
+  for (int side = 0; side < 2; ++side) {
+    float ea[N], eb[N];
+    const float lb = leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + side * RECS, x + side * 2 * G, ea, eb);
+    float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+    MatrixSteps<0, KL, N>::run(ea, eb, side == 0 ? A1 : A2, d0, d1, ea[0] * eb[0], ea[1 / N] * eb[1 % N]);
+    const float m = rmax(rmax(rmax(d0[0], d0[1]), rmax(d0[2], d0[3])), rmax(rmax(d1[0], d1[1]), rmax(d1[2], d1[3])));
+    const float inv = __builtin_amdgcn_rcpf(rmax(m, 0x1p-100f));
+    float* v = side == 0 ? va : vb;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      v[t] = d0[t] * inv;
+      v[4 + t] = d1[t] * inv;
+    }
+    base += lb + Mt::log(m);
+  }
+  matrixChainAndStore<LOG2, SPILL, 8, 8>(va, vb, AT, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
+  return ip + 2 + M + 1 + 4 * G + 2 * RECS + 2 * KL * M + 64 * M;
+}
+template <bool LOG2, bool SPILL, bool TIERED, int N>
+__device__ __forceinline__ code_ptr leafPairMatrixG(code_ptr ip, const Head& h, uint32_t leaves, bool marginal, const float* wGlobal,
+                                                     const Slots<float, SPILL>& S) {
+  if (!marginal) {
+    if (leaves == 2) return leafPairMatrix<LOG2, SPILL, TIERED, N, 2, false>(ip, h, wGlobal, S);
+    if (leaves == 1) return leafPairMatrix<LOG2, SPILL, TIERED, N, 1, false>(ip, h, wGlobal, S);
+    return leafPairMatrix<LOG2, SPILL, TIERED, N, 4, false>(ip, h, wGlobal, S);
+  }
+  if (leaves == 2) return leafPairMatrix<LOG2, SPILL, TIERED, N, 2, true>(ip, h, wGlobal, S);
+  if (leaves == 1) return leafPairMatrix<LOG2, SPILL, TIERED, N, 1, true>(ip, h, wGlobal, S);
+  return leafPairMatrix<LOG2, SPILL, TIERED, N, 4, true>(ip, h, wGlobal, S);
 }
 
 // n products of G Gaussian leaves each. The records are independent, so they are taken four at
@@ -725,6 +806,15 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
   }
   const int na = int((w0 >> 8) & 0xffu), nb = int((w0 >> 16) & 0xffu);
   if constexpr (sizeof(R) == 4) {
+    if (op == OP_LEAFPAIRMM) {
+      // na: operand count per list of the two leaf regions. The weights follow the header words, destinations, scale slot,
+      // 4 G feature slots and the constants of 4 na products of G leaves.
+      const uint32_t leaves = (h.word(2) >> 12) & 0xfu;
+      const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 11 + 4 * leaves + 4 * na * leaves * 3);
+      // Leaf regions of 4x4 products only: with 8x8 the three sets of weights and the operands of two long chains
+      // would cost the whole kernel a wavefront per SIMD in registers; those stay single OP_LEAFMM instructions.
+      return leafPairMatrixG<LOG2, SPILL, TIERED, 4>(ip, h, leaves, a.marginal != 0, wGlobal, S);
+    }
     if (op == OP_LEAFMM) {
       // The weights start after the two header words, eight destinations, the scale slot, the feature slots and the leaf constants.
       const uint32_t leaves = (h.word(2) >> 12) & 0xfu;

@@ -283,6 +283,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   std::vector<bool> matrixInstr(instrs.size(), false);
   std::vector<int> linearConsumer(instrs.size(), -1);  // producer -> consuming instruction
   std::vector<bool> leafRegion(instrs.size(), false), fusedProduct(instrs.size(), false);
+  std::vector<std::pair<uint32_t, uint32_t>> leafPair(instrs.size(), {NONE, NONE});  // 8x8 sum -> the two leaf regions it takes in
   {
     for (uint32_t k = 0; k < instrs.size(); ++k) {
       const Instr& in = instrs[k];
@@ -341,6 +342,23 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       if (!ok || fa.size() != fb.size() || !(fa.size() == 1 || fa.size() == 2 || fa.size() == 4)) continue;
       leafRegion[k] = true;
       for (uint32_t s : instrs[k].srcs) fusedProduct[instrOfNode[s]] = true;
+      instrs[k].srcs.clear();
+    }
+    // Pairs of leaf regions: an 8x8 outer sum whose operand lists are the scaled result vectors of two leaf
+    // regions of 4x4 products each, read by nothing else, takes them in: one instruction, the vectors stay in registers.
+    for (uint32_t k = 0; k < instrs.size() && o.interpLeafRegions; ++k) {
+      if (!matrixInstr[k] || leafRegion[k]) continue;
+      const Outer& outer = outerOf.at(g.nodes[instrs[k].node].children);
+      if (outer.a.size() != 8 || outer.b.size() != 8) continue;
+      const uint32_t i = instrOfNode[outer.a[0]], j = instrOfNode[outer.b[0]];
+      if (i == NONE || j == NONE || i == j || !leafRegion[i] || !leafRegion[j] || linearConsumer[i] != int(k) || linearConsumer[j] != int(k) ||
+          instrs[i].defs != outer.a || instrs[j].defs != outer.b)
+        continue;
+      const Outer& oi = outerOf.at(g.nodes[instrs[i].node].children);
+      const Outer& oj = outerOf.at(g.nodes[instrs[j].node].children);
+      if (oi.a.size() != 4 || oj.a.size() != 4 || g.nodes[oi.a[0]].children.size() != g.nodes[oj.a[0]].children.size()) continue;
+      leafPair[k] = {i, j};
+      fusedProduct[i] = fusedProduct[j] = true;
       instrs[k].srcs.clear();
     }
   }
@@ -625,17 +643,12 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
             if (slotOf[nodes[j]] != slotOf[nodes[0]] + j) return false;
           return true;
         };
-        if (leafRegion[k]) {
-          const uint32_t G = uint32_t(g.nodes[outer.a[0]].children.size());
-          if (stagedLong) longFlag |= 0x80u;
-          b.word(OP_LEAFMM | longFlag | (na << 8) | (nb << 16) | (tierOf(defs) << 28));
-          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | (stagedLong ? 1u << 16 : 0u));
-          for (uint32_t d : defs) slotWord(slotOf[d]);
-          if (scaleDst != NONE) slotWord(scaleDst);
-          else b.word(NONE);
-          for (uint32_t list : {outer.a[0], outer.b[0]})
+        auto emitLeafFeatures = [&](const Outer& region) {
+          for (uint32_t list : {region.a[0], region.b[0]})
             for (uint32_t c : g.nodes[list].children) slotWord(valueSlotOf[g.nodes[c].feature]);
-          for (const std::vector<uint32_t>* list : {&outer.a, &outer.b})
+        };
+        auto emitLeafConstants = [&](const Outer& region) {
+          for (const std::vector<uint32_t>* list : {&region.a, &region.b})
             for (uint32_t prod : *list)
               for (uint32_t c : g.nodes[prod].children) {
                 const auto& leaf = g.nodes[c];
@@ -644,9 +657,47 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
                 b.real(coef / den);
                 b.real(den * b.scale);
               }
-          for (uint32_t grp = 0; grp < na * nb / 16; ++grp)
+        };
+        auto emitMatrixWeights = [&](const std::vector<uint32_t>& sums, uint32_t products) {
+          for (uint32_t grp = 0; grp < products / 16; ++grp)
             for (uint32_t half = 0; half < 2; ++half)
-              for (uint32_t lane = 0; lane < 64; ++lane) b.real(g.nodes[defs[half * 4 + lane % 4]].weights[grp * 16 + lane / 4]);
+              for (uint32_t lane = 0; lane < 64; ++lane) b.real(g.nodes[sums[half * 4 + lane % 4]].weights[grp * 16 + lane / 4]);
+        };
+        if (leafPair[k].first != NONE) {
+          const Instr& ri = instrs[leafPair[k].first];
+          const Instr& rj = instrs[leafPair[k].second];
+          const Outer& oi = outerOf.at(g.nodes[ri.node].children);
+          const Outer& oj = outerOf.at(g.nodes[rj.node].children);
+          const uint32_t N = uint32_t(oi.a.size()), G = uint32_t(g.nodes[oi.a[0]].children.size());
+          if (stagedLong) longFlag |= 0x80u;
+          b.word(OP_LEAFPAIRMM | longFlag | (N << 8) | (tierOf(defs) << 28));
+          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | (stagedLong ? 1u << 16 : 0u));
+          for (uint32_t d : defs) slotWord(slotOf[d]);
+          if (scaleDst != NONE) slotWord(scaleDst);
+          else b.word(NONE);
+          emitLeafFeatures(oi);
+          emitLeafFeatures(oj);
+          emitLeafConstants(oi);
+          emitLeafConstants(oj);
+          emitMatrixWeights(ri.defs, N * N);
+          emitMatrixWeights(rj.defs, N * N);
+          emitMatrixWeights(defs, 64);
+          b.end(at);
+          b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = leafpair(8 sums x 8x8 products of two leaf regions: 8 sums x " << N << "x" << N
+                << " products of " << G << " gaussians)" << (scaleDst != NONE ? " scaled" : "") << "   ; nodes " << in.defs[0] << "..\n";
+          break;
+        }
+        if (leafRegion[k]) {
+          const uint32_t G = uint32_t(g.nodes[outer.a[0]].children.size());
+          if (stagedLong) longFlag |= 0x80u;
+          b.word(OP_LEAFMM | longFlag | (na << 8) | (nb << 16) | (tierOf(defs) << 28));
+          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | (stagedLong ? 1u << 16 : 0u));
+          for (uint32_t d : defs) slotWord(slotOf[d]);
+          if (scaleDst != NONE) slotWord(scaleDst);
+          else b.word(NONE);
+          emitLeafFeatures(outer);
+          emitLeafConstants(outer);
+          emitMatrixWeights(defs, na * nb);
           b.end(at);
           b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = leafregion(8 sums x " << na << "x" << nb << " products of " << G << " gaussians)"
                 << (scaleDst != NONE ? " scaled" : "") << "   ; nodes " << in.defs[0] << "..\n";

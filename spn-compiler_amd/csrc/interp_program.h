@@ -38,6 +38,11 @@ enum InterpOp : uint32_t {
                     //   0xFFFFFFFF), G feature slots of the a list, G of the b list, (NA+NB)*G*(mean, shift, den),
                     //   weights as in OP_OUTERMM: an OP_OUTERMM whose operand lists are products of G Gaussian leaves
                     //   each, all products of a list over the same features; they are computed in registers
+  OP_LEAFPAIRMM = 8,// [op|N<<8|dstTier<<28][8|outScaled<<8|dstRun<<11|G<<12|featTier<<16] dst*8, scaleDst (or 0xFFFFFFFF),
+                    //   feature slots (a and b list of the first leaf region, then of the second: 4 G), constants of the
+                    //   first region's 2 N products and of the second's, weights of the first region (N*N*8), of the
+                    //   second, of the 8x8 sum over the two result vectors (512), each as in OP_OUTERMM: two OP_LEAFMM
+                    //   of N x N products and the OP_OUTERMM over their results in one instruction (emitted for N = 4)
   OP_PRODBATCH = 5, // [op|n<<8][G|featTier<<8|dstTier<<10|grouped<<12] n*(dst, G*(feat, mean, shift, den))
                     //   n products of G Gaussian leaves each; the records are independent of each other.
                     //   Tiers as in OP_OUTERMM (0 short pool, 1 long pool, 2 mixed); grouped: in every full group

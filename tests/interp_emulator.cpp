@@ -215,58 +215,85 @@ int main(int argc, char** argv) {
             for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), base + lg(res[t]));
           }
           pc = w + size_t(na) * nb * M;
-        } else if (op == OP_LEAFMM) {
-          // An outer sum in matrix form whose operands are products of G Gaussian leaves, computed on the spot.
-          const uint32_t na = (w0 >> 8) & 0xff, nb = (w0 >> 16) & 0xff, w1 = c.at(pc + 1), M = w1 & 0xff, G = (w1 >> 12) & 0xf;
+        } else if (op == OP_LEAFMM || op == OP_LEAFPAIRMM) {
+          // OP_LEAFMM: an outer sum in matrix form whose operands are products of G Gaussian leaves, computed on the
+          // spot. OP_LEAFPAIRMM: two of those and the 8x8 outer sum over their (scaled) result vectors.
+          const bool pair = op == OP_LEAFPAIRMM;
+          const uint32_t na = (w0 >> 8) & 0xff, nb = pair ? na : (w0 >> 16) & 0xff, w1 = c.at(pc + 1), M = w1 & 0xff, G = (w1 >> 12) & 0xf;
           const bool outScaled = (w1 >> 8) & 1;
-          if (M != 8 || !((na == 4 && nb == 4) || (na == 8 && nb == 8)) || !(G == 1 || G == 2 || G == 4) || p.featureMode != FEAT_STAGED)
+          if (M != 8 || !((na == 4 && nb == 4) || (na == 8 && nb == 8 && !pair)) || !(G == 1 || G == 2 || G == 4) || p.featureMode != FEAT_STAGED)
             throw std::runtime_error("malformed leaf region at word " + std::to_string(pc));
-          const size_t d0 = pc + 2, sc = d0 + M, f0 = sc + 1, r0 = f0 + 2 * G, w = r0 + size_t(na + nb) * G * 3;
+          const uint32_t regions = pair ? 2 : 1, nf = 2 * G * regions;
+          const size_t d0 = pc + 2, sc = d0 + M, f0 = sc + 1, r0 = f0 + nf, recs = size_t(na + nb) * G * 3, w = r0 + recs * regions;
           uint32_t longDst = 0, longFeat = 0;
           for (uint32_t t = 0; t < M; ++t) longDst += c.at(d0 + t) >= p.shortSlots ? 1 : 0;
-          for (uint32_t j = 0; j < 2 * G; ++j) longFeat += c.at(f0 + j) >= p.shortSlots ? 1 : 0;
-          if (((w0 >> 28) & 3) != (longDst == 0 ? 0u : (longDst == M ? 1u : 2u)) || (longFeat != 0 && longFeat != 2 * G) ||
+          for (uint32_t j = 0; j < nf; ++j) longFeat += c.at(f0 + j) >= p.shortSlots ? 1 : 0;
+          if (((w0 >> 28) & 3) != (longDst == 0 ? 0u : (longDst == M ? 1u : 2u)) || (longFeat != 0 && longFeat != nf) ||
               ((w1 >> 16) & 3) != (longFeat ? 1u : 0u))
             throw std::runtime_error("tier bits disagree with the slot lists at word " + std::to_string(pc));
           if ((w1 >> 11) & 1)
             for (uint32_t t = 1; t < M; ++t)
               if (c.at(d0 + t) != c.at(d0) + t) throw std::runtime_error("run flag on a list of non-consecutive slots at word " + std::to_string(pc));
           if ((c.at(sc) != UINT32_MAX) != outScaled) throw std::runtime_error("scale slot disagrees with the format bit at word " + std::to_string(pc));
-          std::vector<float> e(na + nb);
-          for (uint32_t i = 0; i < na + nb; ++i) {
-            float acc = 0;
-            for (uint32_t j = 0; j < G; ++j) {
-              const size_t q = r0 + (size_t(i) * G + j) * 3;
-              const float xv = rd(c.at(f0 + (i < na ? 0 : G) + j));
-              const float d = xv - asFloat(c.at(q));
-              float v = (d * d + asFloat(c.at(q + 1))) * asFloat(c.at(q + 2));
-              if (g.supportMarginal && xv != xv) v = 0;
-              acc += v;
-            }
-            e[i] = acc;
-          }
-          float ma = -INFINITY, mb = -INFINITY;
-          for (uint32_t r = 0; r < na; ++r) ma = std::fmax(ma, e[r]);
-          for (uint32_t cc = 0; cc < nb; ++cc) mb = std::fmax(mb, e[na + cc]);
-          ma = std::fmax(ma, -3.4028234663852886e38f);
-          mb = std::fmax(mb, -3.4028234663852886e38f);
-          std::vector<float> res(M, 0.f);
-          for (uint32_t t = 0; t < M; ++t)
-            for (uint32_t r = 0; r < na; ++r)
-              for (uint32_t cc = 0; cc < nb; ++cc) {
-                const uint32_t k = r * nb + cc;
-                res[t] += ex(e[r] - ma) * ex(e[na + cc] - mb) * asFloat(c.at(w + (k / 16) * 128 + (t / 4) * 64 + (k % 16) * 4 + t % 4));
+          auto weight = [&](size_t at, uint32_t k, uint32_t t) { return asFloat(c.at(at + (k / 16) * 128 + (t / 4) * 64 + (k % 16) * 4 + t % 4)); };
+          // One leaf region: sums over exp2(product - max) pairs; returns the two maxima's sum.
+          auto leafRegion = [&](size_t feat, size_t rec, size_t wAt, std::vector<float>& res) {
+            std::vector<float> e(na + nb);
+            for (uint32_t i = 0; i < na + nb; ++i) {
+              float acc = 0;
+              for (uint32_t j = 0; j < G; ++j) {
+                const size_t q = rec + (size_t(i) * G + j) * 3;
+                const float xv = rd(c.at(feat + (i < na ? 0 : G) + j));
+                const float d = xv - asFloat(c.at(q));
+                float v = (d * d + asFloat(c.at(q + 1))) * asFloat(c.at(q + 2));
+                if (g.supportMarginal && xv != xv) v = 0;
+                acc += v;
               }
-          if (outScaled) {
+              e[i] = acc;
+            }
+            float ma = -INFINITY, mb = -INFINITY;
+            for (uint32_t r = 0; r < na; ++r) ma = std::fmax(ma, e[r]);
+            for (uint32_t cc = 0; cc < nb; ++cc) mb = std::fmax(mb, e[na + cc]);
+            ma = std::fmax(ma, -3.4028234663852886e38f);
+            mb = std::fmax(mb, -3.4028234663852886e38f);
+            res.assign(M, 0.f);
+            for (uint32_t t = 0; t < M; ++t)
+              for (uint32_t r = 0; r < na; ++r)
+                for (uint32_t cc = 0; cc < nb; ++cc) res[t] += ex(e[r] - ma) * ex(e[na + cc] - mb) * weight(wAt, r * nb + cc, t);
+            return ma + mb;
+          };
+          auto scaled = [&](std::vector<float>& res) {  // res / max(res); returns log2(max)
             float m = 0.f;
             for (uint32_t t = 0; t < M; ++t) m = std::fmax(m, res[t]);
             const float inv = 1.0f / std::fmax(m, 0x1p-100f);
-            for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), res[t] * inv);
-            wr(c.at(sc), ma + mb + lg(m));
+            for (uint32_t t = 0; t < M; ++t) res[t] *= inv;
+            return lg(m);
+          };
+          std::vector<float> res;
+          float base;
+          if (pair) {
+            std::vector<float> va, vb;
+            base = leafRegion(f0, r0, w, va);
+            base += scaled(va);
+            base += leafRegion(f0 + 2 * G, r0 + recs, w + size_t(na) * nb * M, vb);
+            base += scaled(vb);
+            const size_t wt = w + 2 * size_t(na) * nb * M;
+            res.assign(M, 0.f);
+            for (uint32_t t = 0; t < M; ++t)
+              for (uint32_t r = 0; r < 8; ++r)
+                for (uint32_t cc = 0; cc < 8; ++cc) res[t] += va[r] * vb[cc] * weight(wt, r * 8 + cc, t);
+            pc = wt + 64 * M;
           } else {
-            for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), ma + mb + lg(res[t]));
+            base = leafRegion(f0, r0, w, res);
+            pc = w + size_t(na) * nb * M;
           }
-          pc = w + size_t(na) * nb * M;
+          if (outScaled) {
+            const float l = scaled(res);
+            for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), res[t]);
+            wr(c.at(sc), base + l);
+          } else {
+            for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), base + lg(res[t]));
+          }
         } else {
           throw std::runtime_error("unknown opcode at word " + std::to_string(pc));
         }

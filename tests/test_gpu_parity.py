@@ -449,9 +449,10 @@ def test_matrix_form_outer_sums(native, case, marginal):
         assert np.abs(got - want64).max() <= F32_TOL * max(1.0, np.abs(want64).max() / 100), opts
 
 
-def _leaf_region_graph(seed, count, leaves_per_product, regions, marginal):
+def _leaf_region_graph(seed, count, leaves_per_product, regions, marginal, paired=False):
     """Sums over pairs of leaf regions: each leaf region holds `count` products of `leaves_per_product`
-    Gaussians over features of its own; `regions` pairs are combined by outer products and eight sums each."""
+    Gaussians over features of its own; `regions` pairs are combined by outer products and eight sums each.
+    paired: two such sum vectors at a time are combined the same way once more."""
     from spnc.structure import Gaussian, Product, Sum
     rng = np.random.default_rng(seed)
     G = leaves_per_product
@@ -461,14 +462,18 @@ def _leaf_region_graph(seed, count, leaves_per_product, regions, marginal):
         return [Product(children=[Gaussian(mean=float(rng.normal()), stdev=float(rng.uniform(0.3, 1.4)), scope=int(f)) for f in scope])
                 for _ in range(count)]
 
-    tops = []
+    def sums_over(left, right):
+        products = [Product(children=[a, b]) for a in left for b in right]
+        return [Sum(weights=[float(v) for v in rng.dirichlet(np.ones(len(products)))], children=products) for _ in range(8)]
+
+    vectors = []
     for r in range(regions):
         scope = list(range(2 * G * r, 2 * G * (r + 1)))
-        left, right = leaf_region(scope[:G]), leaf_region(scope[G:])
-        products = [Product(children=[a, b]) for a in left for b in right]
-        sums = [Sum(weights=[float(v) for v in rng.dirichlet(np.ones(len(products)))], children=products) for _ in range(8)]
-        tops.append(Sum(weights=[float(v) for v in rng.dirichlet(np.ones(8))], children=sums))
-    spn = Product(children=tops) if regions > 1 else tops[0]
+        vectors.append(sums_over(leaf_region(scope[:G]), leaf_region(scope[G:])))
+    if paired:
+        vectors = [sums_over(vectors[i], vectors[i + 1]) for i in range(0, regions - 1, 2)] + (vectors[-1:] if regions % 2 else [])
+    tops = [Sum(weights=[float(v) for v in rng.dirichlet(np.ones(8))], children=v) for v in vectors]
+    spn = Product(children=tops) if len(tops) > 1 else tops[0]
     X = rng.normal(0, 1.2, (600, num_features))
     if marginal:
         X[rng.random(X.shape) < 0.2] = np.nan
@@ -487,6 +492,25 @@ def test_leaf_regions_inside_the_outer_sum(native, count, leaves, marginal):
                  {"hip-interp-lds-slots": 6}, {"hip-interp-leaf-regions": "false"}):
         k = compile_spn(native, spn, "float64", marginal=marginal, **dict(opts, **{"hip-kernel": "interpreter"}))
         assert ("leafregion(8 sums x" in k.source()) == (opts.get("hip-interp-leaf-regions") != "false"), k.source()[:2000]
+        got = run(k, X)
+        assert got.dtype == np.float32
+        assert np.abs(got - want64).max() <= F32_TOL * max(1.0, np.abs(want64).max() / 100), opts
+
+
+@pytest.mark.parametrize("count,leaves", [(4, 2), (8, 2), (4, 4), (8, 1), (4, 1)])
+@pytest.mark.parametrize("marginal", [False, True])
+def test_pairs_of_leaf_regions_inside_the_outer_sum(native, count, leaves, marginal):
+    """An 8x8 outer sum over the result vectors of two leaf regions takes both in; five leaf regions give two such
+    pairs and one leaf region on its own."""
+    spn, X = _leaf_region_graph(900 + 10 * count + leaves, count, leaves, 5, marginal, paired=True)
+    want64 = ev.ll_closed_f64(oracle_model(spn, "float64"), X, marginal=marginal)
+    for opts in ({}, {"hip-interp-staged-features": "spill", "hip-interp-long-range": 4, "hip-interp-lds-slots": 30},
+                 {"hip-interp-staged-features": "lds", "hip-interp-short-slots": 12, "hip-interp-long-range": 2, "hip-interp-lds-slots": 40},
+                 {"hip-interp-lds-slots": 6}, {"hip-interp-scaled-vectors": "false"}):
+        k = compile_spn(native, spn, "float64", marginal=marginal, **dict(opts, **{"hip-kernel": "interpreter"}))
+        src = k.source()
+        pairs = 2 if count == 4 and "hip-interp-scaled-vectors" not in opts else 0   # only 4x4 leaf regions are taken in as pairs
+        assert src.count("leafpair(") == pairs and src.count("leafregion(") == 5 - 2 * pairs, src[:2000]
         got = run(k, X)
         assert got.dtype == np.float32
         assert np.abs(got - want64).max() <= F32_TOL * max(1.0, np.abs(want64).max() / 100), opts
