@@ -787,13 +787,34 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
       S.wr(dst, S.rd(ip[0]) + constAt<R>(ip, 1));
       return ip + 1 + RW;
     }
-    R m = R(-__builtin_huge_val());
+    // Terms are taken in chunks (sixteen, eight or four), all reads of a chunk in flight together; the running sum is kept
+    // relative to the running maximum and rescaled when a chunk raises it, so every term is read once.
+    constexpr int C = sizeof(R) == 8 ? 4 : (LOG2 ? 16 : 8);  // fewer values in registers where they or the exponentials are large
+    R ms = Mt::lowest(), acc = R(0);
+    int j = 0;
+    for (; j + C <= k; j += C) {
+      R v[C];
+#pragma unroll
+      for (int q = 0; q < C; ++q) v[q] = S.rd(ip[long(j + q) * (1 + RW)]);
+      R cm = v[0];
+#pragma unroll
+      for (int q = 1; q < C; ++q) cm = rmax(cm, v[q]);
+      const R mn = rmax(ms, cm);
+      acc *= Mt::exp(ms - mn);
+      ms = mn;
+#pragma unroll
+      for (int q = 0; q < C; ++q) acc = rfma(Mt::exp(v[q] - ms), constAt<R>(ip, long(j + q) * (1 + RW) + 1), acc);
+    }
+    if (j < k) {
+      R cm = R(-__builtin_huge_val());
 #pragma unroll 4
-    for (int j = 0; j < k; ++j) m = rmax(m, S.rd(ip[long(j) * (1 + RW)]));
-    const R ms = rmax(m, Mt::lowest());
-    R acc = R(0);
+      for (int q = j; q < k; ++q) cm = rmax(cm, S.rd(ip[long(q) * (1 + RW)]));
+      const R mn = rmax(ms, cm);
+      acc *= Mt::exp(ms - mn);
+      ms = mn;
 #pragma unroll 4
-    for (int j = 0; j < k; ++j) acc = rfma(Mt::exp(S.rd(ip[long(j) * (1 + RW)]) - ms), constAt<R>(ip, long(j) * (1 + RW) + 1), acc);
+      for (int q = j; q < k; ++q) acc = rfma(Mt::exp(S.rd(ip[long(q) * (1 + RW)]) - ms), constAt<R>(ip, long(q) * (1 + RW) + 1), acc);
+    }
     S.wr(dst, ms + Mt::log(acc));
     return ip + long(k) * (1 + RW);
   }
@@ -906,6 +927,7 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
         const uint32_t op = w0 & 0x7fu;
         int c = (op == OP_PROD || op == OP_PRODBATCH) ? 0 : (op == OP_OUTERSUM || op == OP_OUTERMM) ? ((((w0 >> 16) & 0xffu) == 8 ? 1 : 2) + (spillPath ? 2 : 0)) : 5;
         if ((op == OP_PROD || op == OP_PRODBATCH) && spillPath) c = 6;
+        if (op == OP_LEAFMM || op == OP_LEAFPAIRMM) c = 7;
 #pragma unroll
         for (int q = 0; q < 8; ++q)
           if (q == c) {
@@ -918,8 +940,8 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
     }
 #ifdef SPN_INTERP_PROFILE
     if (blockIdx.x == 0 && threadIdx.x == 0 && base == 2 * lanes)
-      printf("profile: prod %d/%lld outer8 %d/%lld outer4 %d/%lld outer8-spill %d/%lld outer4-spill %d/%lld other %d/%lld prod-spill %d/%lld\n",
-             cnt[0], cyc[0], cnt[1], cyc[1], cnt[2], cyc[2], cnt[3], cyc[3], cnt[4], cyc[4], cnt[5], cyc[5], cnt[6], cyc[6]);
+      printf("profile: prod %d/%lld outer8 %d/%lld outer4 %d/%lld outer8-spill %d/%lld outer4-spill %d/%lld other %d/%lld prod-spill %d/%lld leaf %d/%lld\n",
+             cnt[0], cyc[0], cnt[1], cyc[1], cnt[2], cyc[2], cnt[3], cyc[3], cnt[4], cyc[4], cnt[5], cyc[5], cnt[6], cyc[6], cnt[7], cyc[7]);
 #endif
     if (valid) out[i] = Mt::finish(result);
   }
