@@ -160,6 +160,7 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
     k->bytesPerResult_ = k->prog_.f64 ? 8 : 4;
     k->inputAlign_ = g.ftype.bytes;
     k->text_ = k->prog_.listing;
+    k->gridPolicy_ = std::max(0, o.blocksPerCU);  // a limit on the resident blocks; the interpreter is always persistent
   } else {
     k->kind_ = SPNC_HIP_KERNEL_JIT;
     JitSource js = emitHipSource(g, o);
@@ -366,6 +367,7 @@ void Kernel::ensureDevice() {
     int nb = 0;
     hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, interpMode_, ldsBytes_, &nb), "occupancy query");
     blocksPerCU_ = std::max(1, nb);
+    if (gridPolicy_ > 0) blocksPerCU_ = std::min(blocksPerCU_, gridPolicy_);  // "hip-blocks-per-cu": fewer than fit
     // The kernel touches the cache lines that follow an instruction's weights, so the stream is padded past its end.
     hipCheck(hipMalloc(&dCode_, prog_.code.size() * 4 + 512), "hipMalloc(program)");
     hipCheck(hipMemset(dCode_, 0, prog_.code.size() * 4 + 512), "program padding");
