@@ -524,12 +524,28 @@ __device__ __forceinline__ code_ptr leafRegionMatrixG(code_ptr ip, const Head& h
   return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 4, true>(ip, h, wGlobal, S);
 }
 
+// The matrix chain over ea[r] * eb[c] with the result kept in registers as a scaled vector: v = acc / max(acc);
+// returns log2(max(acc)).
+template <bool LOG2, int NA, int NB>
+__device__ __forceinline__ float scaledChain(const float* ea, const float* eb, const float (*A)[2], float* v) {
+  typedef Math<float, LOG2> Mt;
+  float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+  MatrixSteps<0, NA * NB, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
+  const float m = rmax(rmax(rmax(d0[0], d0[1]), rmax(d0[2], d0[3])), rmax(rmax(d1[0], d1[1]), rmax(d1[2], d1[3])));
+  const float inv = __builtin_amdgcn_rcpf(rmax(m, 0x1p-100f));
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    v[t] = d0[t] * inv;
+    v[4 + t] = d1[t] * inv;
+  }
+  return Mt::log(m);
+}
+
 // OP_LEAFPAIRMM: an 8x8 outer sum whose operand lists are the result vectors of two leaf regions (N x N products
 // of G Gaussian leaves each, eight sums each; N = 4 is what the program builder emits). The two vectors stay in registers as scaled vectors; all weights,
 // features and constants of the three sums are requested at the start.
 template <bool LOG2, bool SPILL, bool TIERED, int N, int G, bool MARGINAL>
 __device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
-  typedef Math<float, LOG2> Mt;
   constexpr int M = 8, KL = N * N, GL = KL / 16;
   // Head: length, opcode, format, eight destinations, the scale slot, 4 G feature slots. ip points at the opcode.
   constexpr int DST = 3, SCALE = DST + M, FEAT = SCALE + 1, REC = FEAT + 4 * G - 1, RECS = 2 * N * G * 3;
@@ -568,17 +584,7 @@ __device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, c
   for (int side = 0; side < 2; ++side) {
     float ea[N], eb[N];
     const float lb = leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + side * RECS, x + side * 2 * G, ea, eb);
-    float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
-    MatrixSteps<0, KL, N>::run(ea, eb, side == 0 ? A1 : A2, d0, d1, ea[0] * eb[0], ea[1 / N] * eb[1 % N]);
-    const float m = rmax(rmax(rmax(d0[0], d0[1]), rmax(d0[2], d0[3])), rmax(rmax(d1[0], d1[1]), rmax(d1[2], d1[3])));
-    const float inv = __builtin_amdgcn_rcpf(rmax(m, 0x1p-100f));
-    float* v = side == 0 ? va : vb;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      v[t] = d0[t] * inv;
-      v[4 + t] = d1[t] * inv;
-    }
-    base += lb + Mt::log(m);
+    base += lb + scaledChain<LOG2, N, N>(ea, eb, side == 0 ? A1 : A2, side == 0 ? va : vb);
   }
   matrixChainAndStore<LOG2, SPILL, 8, 8>(va, vb, AT, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
   return ip + 2 + M + 1 + 4 * G + 2 * RECS + 2 * KL * M + 64 * M;
@@ -594,6 +600,69 @@ __device__ __forceinline__ code_ptr leafPairMatrixG(code_ptr ip, const Head& h, 
   if (leaves == 2) return leafPairMatrix<LOG2, SPILL, TIERED, N, 2, true>(ip, h, wGlobal, S);
   if (leaves == 1) return leafPairMatrix<LOG2, SPILL, TIERED, N, 1, true>(ip, h, wGlobal, S);
   return leafPairMatrix<LOG2, SPILL, TIERED, N, 4, true>(ip, h, wGlobal, S);
+}
+
+// OP_LEAFQUADMM: two OP_LEAFPAIRMM over 4x4 leaf regions and the 8x8 outer sum over their two result vectors, i.e.
+// seven sums over four leaf regions with every intermediate vector in registers. Weights are requested a stage
+// ahead of the chain that uses them: those of the second pair while the first pair's 8x8 chain runs, those of
+// the final sum while the second pair's runs.
+template <bool LOG2, bool SPILL, bool TIERED, int G, bool MARGINAL>
+__device__ __forceinline__ code_ptr leafQuadMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
+  constexpr int N = 4, M = 8;
+  // Head: length, opcode, format, eight destinations, the scale slot, 8 G feature slots. ip points at the opcode.
+  constexpr int DST = 3, SCALE = DST + M, FEAT = SCALE + 1, REC = FEAT + 8 * G - 1, RECS = 2 * N * G * 3;
+  constexpr int LEAFW = N * N * M, PAIRW = 2 * LEAFW + 64 * M;  // weights: leaf, leaf, 8x8 per pair, then the final 8x8
+  const float* wl = wGlobal + (threadIdx.x & 63u);
+  auto loadLeaf = [&](int at, float (*A)[2]) {
+    A[0][0] = wl[at];
+    A[0][1] = wl[at + 64];
+  };
+  auto loadTop = [&](int at, float (*A)[2]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      A[g][0] = wl[at + g * 128];
+      A[g][1] = wl[at + g * 128 + 64];
+    }
+  };
+  float AL[4][1][2], AT[2][4][2], ATOP[4][2];
+  loadLeaf(0, AL[0]);
+  loadLeaf(LEAFW, AL[1]);
+  const uint32_t w0 = h.word(1), w1 = h.word(2);
+  const uint32_t tierD = TIERED ? (w0 >> 28) & 3u : 2u, tierF = TIERED ? (w1 >> 16) & 3u : 2u;
+  float x[8 * G];
+  if (!SPILL || tierF == 0) {
+#pragma unroll
+    for (int j = 0; j < 8 * G; ++j) x[j] = S.rdLds(h.word(FEAT + j));
+  } else if (tierF == 1) {
+#pragma unroll
+    for (int j = 0; j < 8 * G; ++j) x[j] = S.rdSpill(h.word(FEAT + j));
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8 * G; ++j) x[j] = S.rd(h.word(FEAT + j));
+  }
+  loadTop(2 * LEAFW, AT[0]);
+  float pv[2][M], base = 0.f;
+#pragma unroll
+  for (int pair = 0; pair < 2; ++pair) {
+    float v[2][M];
+#pragma unroll
+    for (int side = 0; side < 2; ++side) {
+      const int region = 2 * pair + side;
+      float ea[N], eb[N];
+      base += leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + region * RECS, x + region * 2 * G, ea, eb);
+      base += scaledChain<LOG2, N, N>(ea, eb, AL[region], v[side]);
+    }
+    if (pair == 0) {
+      loadLeaf(PAIRW, AL[2]);
+      loadLeaf(PAIRW + LEAFW, AL[3]);
+      loadTop(PAIRW + 2 * LEAFW, AT[1]);
+    } else {
+      loadTop(2 * PAIRW, ATOP);
+    }
+    base += scaledChain<LOG2, 8, 8>(v[0], v[1], AT[pair], pv[pair]);
+  }
+  matrixChainAndStore<LOG2, SPILL, 8, 8>(pv[0], pv[1], ATOP, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
+  return ip + 2 + M + 1 + 8 * G + 4 * RECS + 2 * PAIRW + 64 * M;
 }
 
 // n products of G Gaussian leaves each. The records are independent, so they are taken four at
@@ -827,6 +896,18 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
   }
   const int na = int((w0 >> 8) & 0xffu), nb = int((w0 >> 16) & 0xffu);
   if constexpr (sizeof(R) == 4) {
+    if (op == OP_LEAFQUADMM) {
+      // One or two leaves per product (the program builder emits no others). The weights follow the header words,
+      // destinations, scale slot, 8 G feature slots and the constants of 32 products of G leaves.
+      const uint32_t leaves = (h.word(2) >> 12) & 0xfu;
+      const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 11 + 8 * leaves + 32 * leaves * 3);
+      if (!a.marginal) {
+        if (leaves == 2) return leafQuadMatrix<LOG2, SPILL, TIERED, 2, false>(ip, h, wGlobal, S);
+        return leafQuadMatrix<LOG2, SPILL, TIERED, 1, false>(ip, h, wGlobal, S);
+      }
+      if (leaves == 2) return leafQuadMatrix<LOG2, SPILL, TIERED, 2, true>(ip, h, wGlobal, S);
+      return leafQuadMatrix<LOG2, SPILL, TIERED, 1, true>(ip, h, wGlobal, S);
+    }
     if (op == OP_LEAFPAIRMM) {
       // na: operand count per list of the two leaf regions. The weights follow the header words, destinations, scale slot,
       // 4 G feature slots and the constants of 4 na products of G leaves.

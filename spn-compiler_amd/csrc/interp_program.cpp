@@ -284,6 +284,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   std::vector<int> linearConsumer(instrs.size(), -1);  // producer -> consuming instruction
   std::vector<bool> leafRegion(instrs.size(), false), fusedProduct(instrs.size(), false);
   std::vector<std::pair<uint32_t, uint32_t>> leafPair(instrs.size(), {NONE, NONE});  // 8x8 sum -> the two leaf regions it takes in
+  std::vector<std::pair<uint32_t, uint32_t>> leafQuad(instrs.size(), {NONE, NONE});  // 8x8 sum -> the two leaf-region pairs it takes in
   {
     for (uint32_t k = 0; k < instrs.size(); ++k) {
       const Instr& in = instrs[k];
@@ -358,6 +359,25 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       const Outer& oj = outerOf.at(g.nodes[instrs[j].node].children);
       if (oi.a.size() != 4 || oj.a.size() != 4 || g.nodes[oi.a[0]].children.size() != g.nodes[oj.a[0]].children.size()) continue;
       leafPair[k] = {i, j};
+      fusedProduct[i] = fusedProduct[j] = true;
+      instrs[k].srcs.clear();
+    }
+    // And once more: an 8x8 outer sum over the result vectors of two such pairs (one or two leaves per product)
+    // takes both pairs in, seven sums over four leaf regions in one instruction.
+    for (uint32_t k = 0; k < instrs.size() && o.interpLeafRegions; ++k) {
+      if (!matrixInstr[k] || leafRegion[k] || leafPair[k].first != NONE) continue;
+      const Outer& outer = outerOf.at(g.nodes[instrs[k].node].children);
+      if (outer.a.size() != 8 || outer.b.size() != 8) continue;
+      const uint32_t i = instrOfNode[outer.a[0]], j = instrOfNode[outer.b[0]];
+      if (i == NONE || j == NONE || i == j || leafPair[i].first == NONE || leafPair[j].first == NONE || linearConsumer[i] != int(k) ||
+          linearConsumer[j] != int(k) || instrs[i].defs != outer.a || instrs[j].defs != outer.b)
+        continue;
+      auto leavesOf = [&](uint32_t pairInstr) {
+        const Outer& region = outerOf.at(g.nodes[instrs[leafPair[pairInstr].first].node].children);
+        return g.nodes[region.a[0]].children.size();
+      };
+      if (leavesOf(i) != leavesOf(j) || leavesOf(i) > 2) continue;
+      leafQuad[k] = {i, j};
       fusedProduct[i] = fusedProduct[j] = true;
       instrs[k].srcs.clear();
     }
@@ -663,6 +683,36 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
             for (uint32_t half = 0; half < 2; ++half)
               for (uint32_t lane = 0; lane < 64; ++lane) b.real(g.nodes[sums[half * 4 + lane % 4]].weights[grp * 16 + lane / 4]);
         };
+        if (leafQuad[k].first != NONE) {
+          // Regions in the order 1, 2 (first pair), 3, 4 (second pair); weights: region, region, pair sum, twice, then this sum.
+          const uint32_t pairs[2] = {leafQuad[k].first, leafQuad[k].second};
+          const Instr* regionInstr[4];
+          const Outer* region[4];
+          for (int q = 0; q < 2; ++q) {
+            regionInstr[2 * q] = &instrs[leafPair[pairs[q]].first];
+            regionInstr[2 * q + 1] = &instrs[leafPair[pairs[q]].second];
+          }
+          for (int r = 0; r < 4; ++r) region[r] = &outerOf.at(g.nodes[regionInstr[r]->node].children);
+          const uint32_t G = uint32_t(g.nodes[region[0]->a[0]].children.size());
+          if (stagedLong) longFlag |= 0x80u;
+          b.word(OP_LEAFQUADMM | longFlag | (4u << 8) | (tierOf(defs) << 28));
+          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | (stagedLong ? 1u << 16 : 0u));
+          for (uint32_t d : defs) slotWord(slotOf[d]);
+          if (scaleDst != NONE) slotWord(scaleDst);
+          else b.word(NONE);
+          for (int r = 0; r < 4; ++r) emitLeafFeatures(*region[r]);
+          for (int r = 0; r < 4; ++r) emitLeafConstants(*region[r]);
+          for (int q = 0; q < 2; ++q) {
+            emitMatrixWeights(regionInstr[2 * q]->defs, 16);
+            emitMatrixWeights(regionInstr[2 * q + 1]->defs, 16);
+            emitMatrixWeights(instrs[pairs[q]].defs, 64);
+          }
+          emitMatrixWeights(defs, 64);
+          b.end(at);
+          b.txt << "  " << slotName(slotOf[in.defs[0]]) << ".. = leafquad(8 sums x 8x8 products of two pairs of leaf regions: 8 sums x 4x4 products of " << G
+                << " gaussians)" << (scaleDst != NONE ? " scaled" : "") << "   ; nodes " << in.defs[0] << "..\n";
+          break;
+        }
         if (leafPair[k].first != NONE) {
           const Instr& ri = instrs[leafPair[k].first];
           const Instr& rj = instrs[leafPair[k].second];

@@ -43,6 +43,11 @@ enum InterpOp : uint32_t {
                     //   first region's 2 N products and of the second's, weights of the first region (N*N*8), of the
                     //   second, of the 8x8 sum over the two result vectors (512), each as in OP_OUTERMM: two OP_LEAFMM
                     //   of N x N products and the OP_OUTERMM over their results in one instruction (emitted for N = 4)
+  OP_LEAFQUADMM = 9,// [op|4<<8|dstTier<<28][8|outScaled<<8|dstRun<<11|G<<12|featTier<<16] dst*8, scaleDst (or 0xFFFFFFFF),
+                    //   8 G feature slots (leaf regions 1 to 4, a list then b list), the constants of the four regions,
+                    //   weights: region 1, region 2, the 8x8 sum over them, region 3, region 4, the 8x8 sum over them,
+                    //   the 8x8 sum over the two pairs' results: two OP_LEAFPAIRMM and the OP_OUTERMM over their
+                    //   results in one instruction (4x4 leaf regions, G = 1 or 2)
   OP_PRODBATCH = 5, // [op|n<<8][G|featTier<<8|dstTier<<10|grouped<<12] n*(dst, G*(feat, mean, shift, den))
                     //   n products of G Gaussian leaves each; the records are independent of each other.
                     //   Tiers as in OP_OUTERMM (0 short pool, 1 long pool, 2 mixed); grouped: in every full group

@@ -215,15 +215,17 @@ int main(int argc, char** argv) {
             for (uint32_t t = 0; t < M; ++t) wr(c.at(d0 + t), base + lg(res[t]));
           }
           pc = w + size_t(na) * nb * M;
-        } else if (op == OP_LEAFMM || op == OP_LEAFPAIRMM) {
+        } else if (op == OP_LEAFMM || op == OP_LEAFPAIRMM || op == OP_LEAFQUADMM) {
           // OP_LEAFMM: an outer sum in matrix form whose operands are products of G Gaussian leaves, computed on the
           // spot. OP_LEAFPAIRMM: two of those and the 8x8 outer sum over their (scaled) result vectors.
-          const bool pair = op == OP_LEAFPAIRMM;
+          // OP_LEAFQUADMM: two of those pairs and the 8x8 outer sum over their result vectors.
+          const bool quad = op == OP_LEAFQUADMM, pair = op == OP_LEAFPAIRMM || quad;
           const uint32_t na = (w0 >> 8) & 0xff, nb = pair ? na : (w0 >> 16) & 0xff, w1 = c.at(pc + 1), M = w1 & 0xff, G = (w1 >> 12) & 0xf;
           const bool outScaled = (w1 >> 8) & 1;
           if (M != 8 || !((na == 4 && nb == 4) || (na == 8 && nb == 8 && !pair)) || !(G == 1 || G == 2 || G == 4) || p.featureMode != FEAT_STAGED)
             throw std::runtime_error("malformed leaf region at word " + std::to_string(pc));
-          const uint32_t regions = pair ? 2 : 1, nf = 2 * G * regions;
+          if (quad && G > 2) throw std::runtime_error("malformed leaf region at word " + std::to_string(pc));
+          const uint32_t regions = quad ? 4 : (pair ? 2 : 1), nf = 2 * G * regions;
           const size_t d0 = pc + 2, sc = d0 + M, f0 = sc + 1, r0 = f0 + nf, recs = size_t(na + nb) * G * 3, w = r0 + recs * regions;
           uint32_t longDst = 0, longFeat = 0;
           for (uint32_t t = 0; t < M; ++t) longDst += c.at(d0 + t) >= p.shortSlots ? 1 : 0;
@@ -271,18 +273,36 @@ int main(int argc, char** argv) {
           };
           std::vector<float> res;
           float base;
-          if (pair) {
+          // A pair: two leaf regions as scaled vectors and the 8x8 sum over them; weights region, region, sum from wAt.
+          auto leafPairSum = [&](uint32_t firstRegion, size_t wAt, std::vector<float>& out) {
             std::vector<float> va, vb;
-            base = leafRegion(f0, r0, w, va);
-            base += scaled(va);
-            base += leafRegion(f0 + 2 * G, r0 + recs, w + size_t(na) * nb * M, vb);
-            base += scaled(vb);
-            const size_t wt = w + 2 * size_t(na) * nb * M;
+            float bs = leafRegion(f0 + 2 * G * firstRegion, r0 + recs * firstRegion, wAt, va);
+            bs += scaled(va);
+            bs += leafRegion(f0 + 2 * G * (firstRegion + 1), r0 + recs * (firstRegion + 1), wAt + size_t(na) * nb * M, vb);
+            bs += scaled(vb);
+            const size_t wt = wAt + 2 * size_t(na) * nb * M;
+            out.assign(M, 0.f);
+            for (uint32_t t = 0; t < M; ++t)
+              for (uint32_t r = 0; r < 8; ++r)
+                for (uint32_t cc = 0; cc < 8; ++cc) out[t] += va[r] * vb[cc] * weight(wt, r * 8 + cc, t);
+            return bs;
+          };
+          const size_t pairWords = 2 * size_t(na) * nb * M + 64 * M;
+          if (quad) {
+            std::vector<float> pa, pb;
+            base = leafPairSum(0, w, pa);
+            base += scaled(pa);
+            base += leafPairSum(2, w + pairWords, pb);
+            base += scaled(pb);
+            const size_t wt = w + 2 * pairWords;
             res.assign(M, 0.f);
             for (uint32_t t = 0; t < M; ++t)
               for (uint32_t r = 0; r < 8; ++r)
-                for (uint32_t cc = 0; cc < 8; ++cc) res[t] += va[r] * vb[cc] * weight(wt, r * 8 + cc, t);
+                for (uint32_t cc = 0; cc < 8; ++cc) res[t] += pa[r] * pb[cc] * weight(wt, r * 8 + cc, t);
             pc = wt + 64 * M;
+          } else if (pair) {
+            base = leafPairSum(0, w, res);
+            pc = w + pairWords;
           } else {
             base = leafRegion(f0, r0, w, res);
             pc = w + size_t(na) * nb * M;

@@ -452,7 +452,7 @@ def test_matrix_form_outer_sums(native, case, marginal):
 def _leaf_region_graph(seed, count, leaves_per_product, regions, marginal, paired=False):
     """Sums over pairs of leaf regions: each leaf region holds `count` products of `leaves_per_product`
     Gaussians over features of its own; `regions` pairs are combined by outer products and eight sums each.
-    paired: two such sum vectors at a time are combined the same way once more."""
+    paired: two such sum vectors at a time are combined the same way once more (2: and the results again)."""
     from spnc.structure import Gaussian, Product, Sum
     rng = np.random.default_rng(seed)
     G = leaves_per_product
@@ -470,8 +470,8 @@ def _leaf_region_graph(seed, count, leaves_per_product, regions, marginal, paire
     for r in range(regions):
         scope = list(range(2 * G * r, 2 * G * (r + 1)))
         vectors.append(sums_over(leaf_region(scope[:G]), leaf_region(scope[G:])))
-    if paired:
-        vectors = [sums_over(vectors[i], vectors[i + 1]) for i in range(0, regions - 1, 2)] + (vectors[-1:] if regions % 2 else [])
+    for _ in range(int(paired)):
+        vectors = [sums_over(vectors[i], vectors[i + 1]) for i in range(0, len(vectors) - 1, 2)] + (vectors[-1:] if len(vectors) % 2 else [])
     tops = [Sum(weights=[float(v) for v in rng.dirichlet(np.ones(8))], children=v) for v in vectors]
     spn = Product(children=tops) if len(tops) > 1 else tops[0]
     X = rng.normal(0, 1.2, (600, num_features))
@@ -511,6 +511,26 @@ def test_pairs_of_leaf_regions_inside_the_outer_sum(native, count, leaves, margi
         src = k.source()
         pairs = 2 if count == 4 and "hip-interp-scaled-vectors" not in opts else 0   # only 4x4 leaf regions are taken in as pairs
         assert src.count("leafpair(") == pairs and src.count("leafregion(") == 5 - 2 * pairs, src[:2000]
+        got = run(k, X)
+        assert got.dtype == np.float32
+        assert np.abs(got - want64).max() <= F32_TOL * max(1.0, np.abs(want64).max() / 100), opts
+
+
+@pytest.mark.parametrize("count,leaves", [(4, 2), (4, 1), (4, 4), (8, 2)])
+@pytest.mark.parametrize("marginal", [False, True])
+def test_quads_of_leaf_regions_inside_the_outer_sum(native, count, leaves, marginal):
+    """Two levels of 8x8 outer sums over 4x4 leaf regions of one or two leaves per product become one instruction;
+    nine leaf regions give two such quads and one leaf region on its own. Other shapes stop at pairs or single regions."""
+    regions = 5 if leaves == 4 else 9   # at most 48 features are staged, and only staged features are fused
+    spn, X = _leaf_region_graph(1300 + 10 * count + leaves, count, leaves, regions, marginal, paired=2)
+    want64 = ev.ll_closed_f64(oracle_model(spn, "float64"), X, marginal=marginal)
+    for opts in ({}, {"hip-interp-staged-features": "spill", "hip-interp-long-range": 4, "hip-interp-lds-slots": 30},
+                 {"hip-interp-staged-features": "lds", "hip-interp-short-slots": 12, "hip-interp-long-range": 2, "hip-interp-lds-slots": 50},
+                 {"hip-interp-lds-slots": 6}):
+        k = compile_spn(native, spn, "float64", marginal=marginal, **dict(opts, **{"hip-kernel": "interpreter"}))
+        src = k.source()
+        want = {(4, 2): (2, 0, 1), (4, 1): (2, 0, 1), (4, 4): (0, 2, 1), (8, 2): (0, 0, 9)}[(count, leaves)]
+        assert (src.count("leafquad("), src.count("leafpair("), src.count("leafregion(")) == want, src[:2000]
         got = run(k, X)
         assert got.dtype == np.float32
         assert np.abs(got - want64).max() <= F32_TOL * max(1.0, np.abs(want64).max() / 100), opts

@@ -199,10 +199,12 @@ def test_generated_source_variants(native):
     k = compile_spn(native, syn.c4_spn(), "float32")
     src = k.source()
     assert k.info()["kernel_kind"] == 2 and "outersum(8 sums x 8x8 products)" in src
-    # the 80 leaf-region pairs are computed inside the 8x8 outer sums over their results, two at a time: no product
-    # instructions and no 4x4 outer sums at all
-    assert src.count("leafpair(8 sums x 8x8 products of two leaf regions: 8 sums x 4x4 products of 2 gaussians) scaled") == 40
-    assert " = prod(" not in src and "prodbatch" not in src and "leafregion(" not in src and "4x4 products)" not in src
+    # the 160 leaf regions are computed inside the outer sums above them, four at a time with the three 8x8 sums over
+    # them: no product instructions and no 4x4 outer sums at all; 8x8 sums of their own remain above (10 root regions
+    # of two and one more level below them)
+    assert src.count("leafquad(8 sums x 8x8 products of two pairs of leaf regions: 8 sums x 4x4 products of 2 gaussians) scaled") == 20
+    assert src.count("outersum(8 sums x 8x8 products)") == 10
+    assert " = prod(" not in src and "prodbatch" not in src and "leafregion(" not in src and "leafpair(" not in src and "4x4 products)" not in src
     k2 = compile_spn(native, syn.c4_spn(), "float32", **{"hip-interp-leaf-regions": "false"})
     # without that, leaf products come in batches of eight (two leaf regions of four), sorted by feature
     assert k2.source().count("prodbatch(8 products x 2 gaussians) grouped") == 80 and "leafregion" not in k2.source()
