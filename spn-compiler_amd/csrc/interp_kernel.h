@@ -34,7 +34,8 @@ hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain
 // Largest dynamic LDS size a block of the interpreter may request on the current device.
 hipError_t interpreterMaxLds(bool f64, bool log2Domain, size_t* bytes);
 
-// Resident blocks per CU for a given dynamic LDS size.
-hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, size_t ldsBytes, int* blocksPerCU);
+// Resident blocks per CU for a given dynamic LDS size. staged: the program stages its features (args.featureMode
+// == FEAT_STAGED at launch); float kernels are built once per feature mode.
+hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, bool staged, size_t ldsBytes, int* blocksPerCU);
 
 }  // namespace spnc_hip

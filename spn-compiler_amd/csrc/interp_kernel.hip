@@ -479,10 +479,36 @@ __device__ __forceinline__ float leafOperands(code_ptr ip, long rec, const float
   return ma + mb;
 }
 
+// Where the fused leaf instructions take their feature values from: staged slots (LDS, spill tier or either,
+// as the tier says) or, when the program does not stage features, the columns of the sample's input row.
+struct FeatureSource {
+  const void* in;
+  uint32_t type;
+  unsigned long long row;
+};
+template <int COUNT, bool STAGED, bool SPILL>
+__device__ __forceinline__ void readLeafFeatures(const Slots<float, SPILL>& S, const Head& h, int pos, uint32_t tier, const FeatureSource& fs,
+                                                 float* x) {
+  if (!STAGED) {
+#pragma unroll
+    for (int j = 0; j < COUNT; ++j) x[j] = featureValue<float>(fs.in, fs.type, fs.row + h.word(pos + j));
+  } else if (!SPILL || tier == 0) {
+#pragma unroll
+    for (int j = 0; j < COUNT; ++j) x[j] = S.rdLds(h.word(pos + j));
+  } else if (tier == 1) {
+#pragma unroll
+    for (int j = 0; j < COUNT; ++j) x[j] = S.rdSpill(h.word(pos + j));
+  } else {
+#pragma unroll
+    for (int j = 0; j < COUNT; ++j) x[j] = S.rd(h.word(pos + j));
+  }
+}
+
 // OP_LEAFMM: the operand lists are products of G Gaussian leaves, all products of a list over the same G features.
 // Weights, features and leaf constants are requested together; the products stay in registers.
-template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB, int G, bool MARGINAL>
-__device__ __forceinline__ code_ptr leafRegionMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
+template <bool LOG2, bool SPILL, bool TIERED, bool STAGED, int NA, int NB, int G, bool MARGINAL>
+__device__ __forceinline__ code_ptr leafRegionMatrix(code_ptr ip, const Head& h, const float* wGlobal, const FeatureSource& fs,
+                                                  const Slots<float, SPILL>& S) {
   constexpr int M = 8, K = NA * NB, GROUPS = K / 16;
   // Head: length, opcode, format, eight destinations, the scale slot, 2 G feature slots. ip points at the opcode.
   constexpr int DST = 3, SCALE = DST + M, FEAT = SCALE + 1, REC = FEAT + 2 * G - 1;  // REC: offset of the constants from ip
@@ -496,32 +522,23 @@ __device__ __forceinline__ code_ptr leafRegionMatrix(code_ptr ip, const Head& h,
   const uint32_t w0 = h.word(1), w1 = h.word(2);
   const uint32_t tierD = TIERED ? (w0 >> 28) & 3u : 2u, tierF = TIERED ? (w1 >> 16) & 3u : 2u;
   float x[2 * G];
-  if (!SPILL || tierF == 0) {
-#pragma unroll
-    for (int j = 0; j < 2 * G; ++j) x[j] = S.rdLds(h.word(FEAT + j));
-  } else if (tierF == 1) {
-#pragma unroll
-    for (int j = 0; j < 2 * G; ++j) x[j] = S.rdSpill(h.word(FEAT + j));
-  } else {
-#pragma unroll
-    for (int j = 0; j < 2 * G; ++j) x[j] = S.rd(h.word(FEAT + j));
-  }
+  readLeafFeatures<2 * G, STAGED>(S, h, FEAT, tierF, fs, x);
   float ea[NA], eb[NB];
   const float base = leafOperands<LOG2, NA, NB, G, MARGINAL>(ip, REC, x, ea, eb);
   matrixChainAndStore<LOG2, SPILL, NA, NB>(ea, eb, A, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
   return ip + 2 + M + 1 + 2 * G + (NA + NB) * G * 3 + K * M;
 }
-template <bool LOG2, bool SPILL, bool TIERED, int NA, int NB>
+template <bool LOG2, bool SPILL, bool TIERED, bool STAGED, int NA, int NB>
 __device__ __forceinline__ code_ptr leafRegionMatrixG(code_ptr ip, const Head& h, uint32_t leaves, bool marginal, const float* wGlobal,
-                                                       const Slots<float, SPILL>& S) {
+                                                       const FeatureSource& fs, const Slots<float, SPILL>& S) {
   if (!marginal) {
-    if (leaves == 2) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 2, false>(ip, h, wGlobal, S);
-    if (leaves == 1) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 1, false>(ip, h, wGlobal, S);
-    return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 4, false>(ip, h, wGlobal, S);
+    if (leaves == 2) return leafRegionMatrix<LOG2, SPILL, TIERED, STAGED, NA, NB, 2, false>(ip, h, wGlobal, fs, S);
+    if (leaves == 1) return leafRegionMatrix<LOG2, SPILL, TIERED, STAGED, NA, NB, 1, false>(ip, h, wGlobal, fs, S);
+    return leafRegionMatrix<LOG2, SPILL, TIERED, STAGED, NA, NB, 4, false>(ip, h, wGlobal, fs, S);
   }
-  if (leaves == 2) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 2, true>(ip, h, wGlobal, S);
-  if (leaves == 1) return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 1, true>(ip, h, wGlobal, S);
-  return leafRegionMatrix<LOG2, SPILL, TIERED, NA, NB, 4, true>(ip, h, wGlobal, S);
+  if (leaves == 2) return leafRegionMatrix<LOG2, SPILL, TIERED, STAGED, NA, NB, 2, true>(ip, h, wGlobal, fs, S);
+  if (leaves == 1) return leafRegionMatrix<LOG2, SPILL, TIERED, STAGED, NA, NB, 1, true>(ip, h, wGlobal, fs, S);
+  return leafRegionMatrix<LOG2, SPILL, TIERED, STAGED, NA, NB, 4, true>(ip, h, wGlobal, fs, S);
 }
 
 // The matrix chain over ea[r] * eb[c] with the result kept in registers as a scaled vector: v = acc / max(acc);
@@ -544,8 +561,9 @@ __device__ __forceinline__ float scaledChain(const float* ea, const float* eb, c
 // OP_LEAFPAIRMM: an 8x8 outer sum whose operand lists are the result vectors of two leaf regions (N x N products
 // of G Gaussian leaves each, eight sums each; N = 4 is what the program builder emits). The two vectors stay in registers as scaled vectors; all weights,
 // features and constants of the three sums are requested at the start.
-template <bool LOG2, bool SPILL, bool TIERED, int N, int G, bool MARGINAL>
-__device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
+template <bool LOG2, bool SPILL, bool TIERED, bool STAGED, int N, int G, bool MARGINAL>
+__device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, const float* wGlobal, const FeatureSource& fs,
+                                                const Slots<float, SPILL>& S) {
   constexpr int M = 8, KL = N * N, GL = KL / 16;
   // Head: length, opcode, format, eight destinations, the scale slot, 4 G feature slots. ip points at the opcode.
   constexpr int DST = 3, SCALE = DST + M, FEAT = SCALE + 1, REC = FEAT + 4 * G - 1, RECS = 2 * N * G * 3;
@@ -564,16 +582,7 @@ __device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, c
   const uint32_t w0 = h.word(1), w1 = h.word(2);
   const uint32_t tierD = TIERED ? (w0 >> 28) & 3u : 2u, tierF = TIERED ? (w1 >> 16) & 3u : 2u;
   float x[4 * G];
-  if (!SPILL || tierF == 0) {
-#pragma unroll
-    for (int j = 0; j < 4 * G; ++j) x[j] = S.rdLds(h.word(FEAT + j));
-  } else if (tierF == 1) {
-#pragma unroll
-    for (int j = 0; j < 4 * G; ++j) x[j] = S.rdSpill(h.word(FEAT + j));
-  } else {
-#pragma unroll
-    for (int j = 0; j < 4 * G; ++j) x[j] = S.rd(h.word(FEAT + j));
-  }
+  readLeafFeatures<4 * G, STAGED>(S, h, FEAT, tierF, fs, x);
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     AT[g][0] = wl[2 * KL * M + g * 128];
@@ -589,25 +598,26 @@ __device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, c
   matrixChainAndStore<LOG2, SPILL, 8, 8>(va, vb, AT, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
   return ip + 2 + M + 1 + 4 * G + 2 * RECS + 2 * KL * M + 64 * M;
 }
-template <bool LOG2, bool SPILL, bool TIERED, int N>
+template <bool LOG2, bool SPILL, bool TIERED, bool STAGED, int N>
 __device__ __forceinline__ code_ptr leafPairMatrixG(code_ptr ip, const Head& h, uint32_t leaves, bool marginal, const float* wGlobal,
-                                                     const Slots<float, SPILL>& S) {
+                                                     const FeatureSource& fs, const Slots<float, SPILL>& S) {
   if (!marginal) {
-    if (leaves == 2) return leafPairMatrix<LOG2, SPILL, TIERED, N, 2, false>(ip, h, wGlobal, S);
-    if (leaves == 1) return leafPairMatrix<LOG2, SPILL, TIERED, N, 1, false>(ip, h, wGlobal, S);
-    return leafPairMatrix<LOG2, SPILL, TIERED, N, 4, false>(ip, h, wGlobal, S);
+    if (leaves == 2) return leafPairMatrix<LOG2, SPILL, TIERED, STAGED, N, 2, false>(ip, h, wGlobal, fs, S);
+    if (leaves == 1) return leafPairMatrix<LOG2, SPILL, TIERED, STAGED, N, 1, false>(ip, h, wGlobal, fs, S);
+    return leafPairMatrix<LOG2, SPILL, TIERED, STAGED, N, 4, false>(ip, h, wGlobal, fs, S);
   }
-  if (leaves == 2) return leafPairMatrix<LOG2, SPILL, TIERED, N, 2, true>(ip, h, wGlobal, S);
-  if (leaves == 1) return leafPairMatrix<LOG2, SPILL, TIERED, N, 1, true>(ip, h, wGlobal, S);
-  return leafPairMatrix<LOG2, SPILL, TIERED, N, 4, true>(ip, h, wGlobal, S);
+  if (leaves == 2) return leafPairMatrix<LOG2, SPILL, TIERED, STAGED, N, 2, true>(ip, h, wGlobal, fs, S);
+  if (leaves == 1) return leafPairMatrix<LOG2, SPILL, TIERED, STAGED, N, 1, true>(ip, h, wGlobal, fs, S);
+  return leafPairMatrix<LOG2, SPILL, TIERED, STAGED, N, 4, true>(ip, h, wGlobal, fs, S);
 }
 
 // OP_LEAFQUADMM: two OP_LEAFPAIRMM over 4x4 leaf regions and the 8x8 outer sum over their two result vectors, i.e.
 // seven sums over four leaf regions with every intermediate vector in registers. Weights are requested a stage
 // ahead of the chain that uses them: those of the second pair while the first pair's 8x8 chain runs, those of
 // the final sum while the second pair's runs.
-template <bool LOG2, bool SPILL, bool TIERED, int G, bool MARGINAL>
-__device__ __forceinline__ code_ptr leafQuadMatrix(code_ptr ip, const Head& h, const float* wGlobal, const Slots<float, SPILL>& S) {
+template <bool LOG2, bool SPILL, bool TIERED, bool STAGED, int G, bool MARGINAL>
+__device__ __forceinline__ code_ptr leafQuadMatrix(code_ptr ip, const Head& h, const float* wGlobal, const FeatureSource& fs,
+                                                const Slots<float, SPILL>& S) {
   constexpr int N = 4, M = 8;
   // Head: length, opcode, format, eight destinations, the scale slot, 8 G feature slots. ip points at the opcode.
   constexpr int DST = 3, SCALE = DST + M, FEAT = SCALE + 1, REC = FEAT + 8 * G - 1, RECS = 2 * N * G * 3;
@@ -630,16 +640,7 @@ __device__ __forceinline__ code_ptr leafQuadMatrix(code_ptr ip, const Head& h, c
   const uint32_t w0 = h.word(1), w1 = h.word(2);
   const uint32_t tierD = TIERED ? (w0 >> 28) & 3u : 2u, tierF = TIERED ? (w1 >> 16) & 3u : 2u;
   float x[8 * G];
-  if (!SPILL || tierF == 0) {
-#pragma unroll
-    for (int j = 0; j < 8 * G; ++j) x[j] = S.rdLds(h.word(FEAT + j));
-  } else if (tierF == 1) {
-#pragma unroll
-    for (int j = 0; j < 8 * G; ++j) x[j] = S.rdSpill(h.word(FEAT + j));
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8 * G; ++j) x[j] = S.rd(h.word(FEAT + j));
-  }
+  readLeafFeatures<8 * G, STAGED>(S, h, FEAT, tierF, fs, x);
   loadTop(2 * LEAFW, AT[0]);
   float pv[2][M], base = 0.f;
 #pragma unroll
@@ -663,6 +664,37 @@ __device__ __forceinline__ code_ptr leafQuadMatrix(code_ptr ip, const Head& h, c
   }
   matrixChainAndStore<LOG2, SPILL, 8, 8>(pv[0], pv[1], ATOP, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
   return ip + 2 + M + 1 + 8 * G + 4 * RECS + 2 * PAIRW + 64 * M;
+}
+
+// The three fused leaf instructions. STAGED: their feature fields are slots of staged values, else input columns.
+template <bool LOG2, bool SPILL, bool TIERED, bool STAGED>
+__device__ __forceinline__ code_ptr leafInstruction(uint32_t op, code_ptr ip, const Head& h, int na, int nb, bool marginal, code_ptr code0,
+                                                    const uint32_t* codeGlobal, const FeatureSource& fs, const Slots<float, SPILL>& S) {
+  const uint32_t leaves = (h.word(2) >> 12) & 0xfu;
+  const float* code = reinterpret_cast<const float*>(codeGlobal) + (ip - code0);
+  if (op == OP_LEAFQUADMM) {
+    // One or two leaves per product (the program builder emits no others). The weights follow the header words,
+    // destinations, scale slot, 8 G feature fields and the constants of 32 products of G leaves.
+    const float* wGlobal = code + (11 + 8 * leaves + 32 * leaves * 3);
+    if (!marginal) {
+      if (leaves == 2) return leafQuadMatrix<LOG2, SPILL, TIERED, STAGED, 2, false>(ip, h, wGlobal, fs, S);
+      return leafQuadMatrix<LOG2, SPILL, TIERED, STAGED, 1, false>(ip, h, wGlobal, fs, S);
+    }
+    if (leaves == 2) return leafQuadMatrix<LOG2, SPILL, TIERED, STAGED, 2, true>(ip, h, wGlobal, fs, S);
+    return leafQuadMatrix<LOG2, SPILL, TIERED, STAGED, 1, true>(ip, h, wGlobal, fs, S);
+  }
+  if (op == OP_LEAFPAIRMM) {
+    // na: operand count per list of the two leaf regions. The weights follow the header words, destinations, scale slot,
+    // 4 G feature fields and the constants of 4 na products of G leaves. Leaf regions of 4x4 products only: with 8x8
+    // the three sets of weights and the operands of two long chains would cost the whole kernel a wavefront per SIMD
+    // in registers; those stay single OP_LEAFMM instructions.
+    const float* wGlobal = code + (11 + 4 * leaves + 4 * na * leaves * 3);
+    return leafPairMatrixG<LOG2, SPILL, TIERED, STAGED, 4>(ip, h, leaves, marginal, wGlobal, fs, S);
+  }
+  // OP_LEAFMM: the weights start after the two header words, eight destinations, the scale slot, the feature fields and the leaf constants.
+  const float* wGlobal = code + (11 + 2 * leaves + (na + nb) * leaves * 3);
+  if (na == 4) return leafRegionMatrixG<LOG2, SPILL, TIERED, STAGED, 4, 4>(ip, h, leaves, marginal, wGlobal, fs, S);
+  return leafRegionMatrixG<LOG2, SPILL, TIERED, STAGED, 8, 8>(ip, h, leaves, marginal, wGlobal, fs, S);
 }
 
 // n products of G Gaussian leaves each. The records are independent, so they are taken four at
@@ -896,33 +928,10 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
   }
   const int na = int((w0 >> 8) & 0xffu), nb = int((w0 >> 16) & 0xffu);
   if constexpr (sizeof(R) == 4) {
-    if (op == OP_LEAFQUADMM) {
-      // One or two leaves per product (the program builder emits no others). The weights follow the header words,
-      // destinations, scale slot, 8 G feature slots and the constants of 32 products of G leaves.
-      const uint32_t leaves = (h.word(2) >> 12) & 0xfu;
-      const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 11 + 8 * leaves + 32 * leaves * 3);
-      if (!a.marginal) {
-        if (leaves == 2) return leafQuadMatrix<LOG2, SPILL, TIERED, 2, false>(ip, h, wGlobal, S);
-        return leafQuadMatrix<LOG2, SPILL, TIERED, 1, false>(ip, h, wGlobal, S);
-      }
-      if (leaves == 2) return leafQuadMatrix<LOG2, SPILL, TIERED, 2, true>(ip, h, wGlobal, S);
-      return leafQuadMatrix<LOG2, SPILL, TIERED, 1, true>(ip, h, wGlobal, S);
-    }
-    if (op == OP_LEAFPAIRMM) {
-      // na: operand count per list of the two leaf regions. The weights follow the header words, destinations, scale slot,
-      // 4 G feature slots and the constants of 4 na products of G leaves.
-      const uint32_t leaves = (h.word(2) >> 12) & 0xfu;
-      const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 11 + 4 * leaves + 4 * na * leaves * 3);
-      // Leaf regions of 4x4 products only: with 8x8 the three sets of weights and the operands of two long chains
-      // would cost the whole kernel a wavefront per SIMD in registers; those stay single OP_LEAFMM instructions.
-      return leafPairMatrixG<LOG2, SPILL, TIERED, 4>(ip, h, leaves, a.marginal != 0, wGlobal, S);
-    }
-    if (op == OP_LEAFMM) {
-      // The weights start after the two header words, eight destinations, the scale slot, the feature slots and the leaf constants.
-      const uint32_t leaves = (h.word(2) >> 12) & 0xfu;
-      const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 11 + 2 * leaves + (na + nb) * leaves * 3);
-      if (na == 4) return leafRegionMatrixG<LOG2, SPILL, TIERED, 4, 4>(ip, h, leaves, a.marginal != 0, wGlobal, S);
-      return leafRegionMatrixG<LOG2, SPILL, TIERED, 8, 8>(ip, h, leaves, a.marginal != 0, wGlobal, S);
+    if (op == OP_LEAFQUADMM || op == OP_LEAFPAIRMM || op == OP_LEAFMM) {
+      const FeatureSource fs{a.in, a.featureType, row};
+      if (stagedMode) return leafInstruction<LOG2, SPILL, TIERED, true>(op, ip, h, na, nb, a.marginal != 0, code0, codeGlobal, fs, S);
+      return leafInstruction<LOG2, SPILL, TIERED, false>(op, ip, h, na, nb, a.marginal != 0, code0, codeGlobal, fs, S);
     }
     if (op == OP_OUTERMM) {
       // The weights start after the two header words, eight destinations, na + nb operands and three scale slots.
@@ -940,7 +949,9 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
 // MODE 0: every slot lives in LDS. MODE 1: slots below ldsSlots (the program's short pool) live
 // in LDS, and only instructions flagged with bit 7 may touch the spill tier. MODE 2: any
 // instruction may touch the spill tier (the short pool did not fit into LDS).
-template <typename R, bool LOG2, int MODE>
+// FEAT 1: the program stages its features in slots; 0: instructions read the input row themselves; 2: either,
+// decided by the launch arguments (one kernel then carries both forms of every instruction that reads features).
+template <typename R, bool LOG2, int MODE, int FEAT>
 __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t* __restrict__ codeGlobal, InterpLaunch a) {
   typedef Math<R, LOG2> Mt;
   extern __shared__ __align__(16) unsigned char ldsRaw[];
@@ -960,7 +971,7 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
   Sl.spillBlock = Sg.spillBlock;
   Sl.ldsSlots = Sg.ldsSlots;
   const unsigned long long F = a.numFeatures;
-  const bool stagedMode = a.featureMode == FEAT_STAGED;
+  const bool stagedMode = FEAT == 2 ? a.featureMode == FEAT_STAGED : FEAT == 1;
 
   for (unsigned long long base = (unsigned long long)blockIdx.x * B; base < a.n; base += lanes) {
     const unsigned long long i = base + threadIdx.x;
@@ -1028,16 +1039,19 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
   }
 }
 
-template <typename R, bool LOG2>
+template <typename R, bool LOG2, int FEAT>
 const void* kernelPtr(int mode) {
-  if (mode == 0) return reinterpret_cast<const void*>(&spn_interp_kernel<R, LOG2, 0>);
-  if (mode == 1) return reinterpret_cast<const void*>(&spn_interp_kernel<R, LOG2, 1>);
-  return reinterpret_cast<const void*>(&spn_interp_kernel<R, LOG2, 2>);
+  if (mode == 0) return reinterpret_cast<const void*>(&spn_interp_kernel<R, LOG2, 0, FEAT>);
+  if (mode == 1) return reinterpret_cast<const void*>(&spn_interp_kernel<R, LOG2, 1, FEAT>);
+  return reinterpret_cast<const void*>(&spn_interp_kernel<R, LOG2, 2, FEAT>);
 }
 
-const void* pick(bool f64, bool log2Domain, int mode) {
-  if (f64) return kernelPtr<double, false>(mode);
-  return log2Domain ? kernelPtr<float, true>(mode) : kernelPtr<float, false>(mode);
+// float kernels exist once per feature mode: the fused leaf instructions are long, and a kernel that held both
+// of their forms would run the staged one slower (instruction fetch). double kernels decide at run time.
+const void* pick(bool f64, bool log2Domain, int mode, bool staged) {
+  if (f64) return kernelPtr<double, false, 2>(mode);
+  if (staged) return log2Domain ? kernelPtr<float, true, 1>(mode) : kernelPtr<float, false, 1>(mode);
+  return log2Domain ? kernelPtr<float, true, 0>(mode) : kernelPtr<float, false, 0>(mode);
 }
 
 }  // namespace
@@ -1054,8 +1068,8 @@ hipError_t interpreterMaxLds(bool f64, bool log2Domain, size_t* bytes) {
   return hipSuccess;
 }
 
-hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, size_t ldsBytes, int* blocksPerCU) {
-  const void* fn = pick(f64, log2Domain, mode);
+hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, bool staged, size_t ldsBytes, int* blocksPerCU) {
+  const void* fn = pick(f64, log2Domain, mode, staged);
   if (ldsBytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(ldsBytes));
     if (e != hipSuccess) return e;
@@ -1065,7 +1079,7 @@ hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, size_t ldsB
 
 hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain, int mode, unsigned grid, size_t ldsBytes,
                              hipStream_t stream) {
-  const void* fn = pick(f64, log2Domain, mode);
+  const void* fn = pick(f64, log2Domain, mode, args.featureMode == FEAT_STAGED);
   if (ldsBytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(ldsBytes));
     if (e != hipSuccess) return e;

@@ -326,7 +326,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       }
       return true;
     };
-    for (uint32_t k = 0; k < instrs.size() && o.interpLeafRegions && p.featureMode == FEAT_STAGED; ++k) {
+    for (uint32_t k = 0; k < instrs.size() && o.interpLeafRegions; ++k) {
       if (!matrixInstr[k]) continue;
       const Outer& outer = outerOf.at(g.nodes[instrs[k].node].children);
       if (!((outer.a.size() == 4 && outer.b.size() == 4) || (outer.a.size() == 8 && outer.b.size() == 8))) continue;
@@ -663,9 +663,15 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
             if (slotOf[nodes[j]] != slotOf[nodes[0]] + j) return false;
           return true;
         };
+        // Feature fields: slots of the staged values, or input columns when features are not staged.
+        const bool stagedFeatures = p.featureMode == FEAT_STAGED;
+        const uint32_t leafFlag = stagedFeatures && stagedLong ? 0x80u : 0u, featTier = stagedFeatures && stagedLong ? 1u << 16 : 0u;
         auto emitLeafFeatures = [&](const Outer& region) {
           for (uint32_t list : {region.a[0], region.b[0]})
-            for (uint32_t c : g.nodes[list].children) slotWord(valueSlotOf[g.nodes[c].feature]);
+            for (uint32_t c : g.nodes[list].children) {
+              if (stagedFeatures) slotWord(valueSlotOf[g.nodes[c].feature]);
+              else b.word(g.nodes[c].feature);
+            }
         };
         auto emitLeafConstants = [&](const Outer& region) {
           for (const std::vector<uint32_t>* list : {&region.a, &region.b})
@@ -694,9 +700,9 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
           }
           for (int r = 0; r < 4; ++r) region[r] = &outerOf.at(g.nodes[regionInstr[r]->node].children);
           const uint32_t G = uint32_t(g.nodes[region[0]->a[0]].children.size());
-          if (stagedLong) longFlag |= 0x80u;
+          longFlag |= leafFlag;
           b.word(OP_LEAFQUADMM | longFlag | (4u << 8) | (tierOf(defs) << 28));
-          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | (stagedLong ? 1u << 16 : 0u));
+          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | featTier);
           for (uint32_t d : defs) slotWord(slotOf[d]);
           if (scaleDst != NONE) slotWord(scaleDst);
           else b.word(NONE);
@@ -719,9 +725,9 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
           const Outer& oi = outerOf.at(g.nodes[ri.node].children);
           const Outer& oj = outerOf.at(g.nodes[rj.node].children);
           const uint32_t N = uint32_t(oi.a.size()), G = uint32_t(g.nodes[oi.a[0]].children.size());
-          if (stagedLong) longFlag |= 0x80u;
+          longFlag |= leafFlag;
           b.word(OP_LEAFPAIRMM | longFlag | (N << 8) | (tierOf(defs) << 28));
-          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | (stagedLong ? 1u << 16 : 0u));
+          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | featTier);
           for (uint32_t d : defs) slotWord(slotOf[d]);
           if (scaleDst != NONE) slotWord(scaleDst);
           else b.word(NONE);
@@ -739,9 +745,9 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
         }
         if (leafRegion[k]) {
           const uint32_t G = uint32_t(g.nodes[outer.a[0]].children.size());
-          if (stagedLong) longFlag |= 0x80u;
+          longFlag |= leafFlag;
           b.word(OP_LEAFMM | longFlag | (na << 8) | (nb << 16) | (tierOf(defs) << 28));
-          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | (stagedLong ? 1u << 16 : 0u));
+          b.word(8u | (scaleDst != NONE ? 0x100u : 0u) | (consecutive(defs) ? 0x800u : 0u) | (G << 12) | featTier);
           for (uint32_t d : defs) slotWord(slotOf[d]);
           if (scaleDst != NONE) slotWord(scaleDst);
           else b.word(NONE);

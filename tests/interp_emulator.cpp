@@ -222,14 +222,15 @@ int main(int argc, char** argv) {
           const bool quad = op == OP_LEAFQUADMM, pair = op == OP_LEAFPAIRMM || quad;
           const uint32_t na = (w0 >> 8) & 0xff, nb = pair ? na : (w0 >> 16) & 0xff, w1 = c.at(pc + 1), M = w1 & 0xff, G = (w1 >> 12) & 0xf;
           const bool outScaled = (w1 >> 8) & 1;
-          if (M != 8 || !((na == 4 && nb == 4) || (na == 8 && nb == 8 && !pair)) || !(G == 1 || G == 2 || G == 4) || p.featureMode != FEAT_STAGED)
+          if (M != 8 || !((na == 4 && nb == 4) || (na == 8 && nb == 8 && !pair)) || !(G == 1 || G == 2 || G == 4))
             throw std::runtime_error("malformed leaf region at word " + std::to_string(pc));
           if (quad && G > 2) throw std::runtime_error("malformed leaf region at word " + std::to_string(pc));
           const uint32_t regions = quad ? 4 : (pair ? 2 : 1), nf = 2 * G * regions;
           const size_t d0 = pc + 2, sc = d0 + M, f0 = sc + 1, r0 = f0 + nf, recs = size_t(na + nb) * G * 3, w = r0 + recs * regions;
           uint32_t longDst = 0, longFeat = 0;
           for (uint32_t t = 0; t < M; ++t) longDst += c.at(d0 + t) >= p.shortSlots ? 1 : 0;
-          for (uint32_t j = 0; j < nf; ++j) longFeat += c.at(f0 + j) >= p.shortSlots ? 1 : 0;
+          const bool stagedFeatures = p.featureMode == FEAT_STAGED;  // else the feature fields are input columns
+          for (uint32_t j = 0; j < nf && stagedFeatures; ++j) longFeat += c.at(f0 + j) >= p.shortSlots ? 1 : 0;
           if (((w0 >> 28) & 3) != (longDst == 0 ? 0u : (longDst == M ? 1u : 2u)) || (longFeat != 0 && longFeat != nf) ||
               ((w1 >> 16) & 3) != (longFeat ? 1u : 0u))
             throw std::runtime_error("tier bits disagree with the slot lists at word " + std::to_string(pc));
@@ -245,7 +246,8 @@ int main(int argc, char** argv) {
               float acc = 0;
               for (uint32_t j = 0; j < G; ++j) {
                 const size_t q = rec + (size_t(i) * G + j) * 3;
-                const float xv = rd(c.at(feat + (i < na ? 0 : G) + j));
+                const uint32_t fw = c.at(feat + (i < na ? 0 : G) + j);
+                const float xv = stagedFeatures ? rd(fw) : float(x[fw]);
                 const float d = xv - asFloat(c.at(q));
                 float v = (d * d + asFloat(c.at(q + 1))) * asFloat(c.at(q + 2));
                 if (g.supportMarginal && xv != xv) v = 0;

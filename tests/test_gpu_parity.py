@@ -516,22 +516,26 @@ def test_pairs_of_leaf_regions_inside_the_outer_sum(native, count, leaves, margi
         assert np.abs(got - want64).max() <= F32_TOL * max(1.0, np.abs(want64).max() / 100), opts
 
 
-@pytest.mark.parametrize("count,leaves", [(4, 2), (4, 1), (4, 4), (8, 2)])
+@pytest.mark.parametrize("count,leaves,regions,want", [
+    (4, 2, 9, (2, 0, 1)), (4, 1, 9, (2, 0, 1)),
+    (4, 4, 5, (0, 2, 1)),     # four leaves per product: pairs, no quads
+    (8, 2, 9, (0, 0, 9)),     # 8x8 leaf regions stay single
+    (4, 2, 13, (3, 0, 1)),    # 52 features: not staged, the fused instructions read the input row
+    (4, 4, 9, (0, 4, 1)),     # 72 features, likewise
+])
 @pytest.mark.parametrize("marginal", [False, True])
-def test_quads_of_leaf_regions_inside_the_outer_sum(native, count, leaves, marginal):
-    """Two levels of 8x8 outer sums over 4x4 leaf regions of one or two leaves per product become one instruction;
-    nine leaf regions give two such quads and one leaf region on its own. Other shapes stop at pairs or single regions."""
-    regions = 5 if leaves == 4 else 9   # at most 48 features are staged, and only staged features are fused
-    spn, X = _leaf_region_graph(1300 + 10 * count + leaves, count, leaves, regions, marginal, paired=2)
+def test_quads_of_leaf_regions_inside_the_outer_sum(native, count, leaves, regions, want, marginal):
+    """Two levels of 8x8 outer sums over 4x4 leaf regions of one or two leaves per product become one instruction
+    (`want`: instructions over four, two and one leaf region); other shapes stop at pairs or single regions."""
+    spn, X = _leaf_region_graph(1300 + 10 * count + leaves + regions, count, leaves, regions, marginal, paired=2)
     want64 = ev.ll_closed_f64(oracle_model(spn, "float64"), X, marginal=marginal)
     for opts in ({}, {"hip-interp-staged-features": "spill", "hip-interp-long-range": 4, "hip-interp-lds-slots": 30},
                  {"hip-interp-staged-features": "lds", "hip-interp-short-slots": 12, "hip-interp-long-range": 2, "hip-interp-lds-slots": 50},
                  {"hip-interp-lds-slots": 6}):
         k = compile_spn(native, spn, "float64", marginal=marginal, **dict(opts, **{"hip-kernel": "interpreter"}))
         src = k.source()
-        want = {(4, 2): (2, 0, 1), (4, 1): (2, 0, 1), (4, 4): (0, 2, 1), (8, 2): (0, 0, 9)}[(count, leaves)]
+        assert ("features direct" in src) == (2 * leaves * regions > 48)
         assert (src.count("leafquad("), src.count("leafpair("), src.count("leafregion(")) == want, src[:2000]
         got = run(k, X)
         assert got.dtype == np.float32
         assert np.abs(got - want64).max() <= F32_TOL * max(1.0, np.abs(want64).max() / 100), opts
-
