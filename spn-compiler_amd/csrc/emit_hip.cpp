@@ -488,35 +488,50 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   const char* mathAttr = inlineMath ? "__forceinline__" : "__attribute__((noinline))";
   if (e.log2Dom && e.f64) {
     // Base-2 exponential and logarithm in double for the arguments this kernel produces (exponents <= 0 up to
-    // rounding, logarithms of sums in [1, fan-in] or of exactly 0): about 20 and 35 instructions where the
-    // general library routines take 40 and 95. exp2: 2^x = 2^n * 2^f, n = rint(x), |f| <= 1/2, 2^f by its Taylor
-    // series to degree 13 (remainder 4e-18). log2: x = 2^e * t, t in [sqrt(1/2), sqrt(2)), z = (t-1)/(t+1),
-    // log2 t = (2/ln 2) z (1 + z^2/3 + ... + z^18/19) (|z| <= 0.172, next term 2e-17). Both agree with the
-    // library to 5e-16 relative over their ranges (checked on the CPU against exp2/log2 of libm).
+    // rounding, logarithms of sums in [1, fan-in] or of exactly 0), by table and short polynomial: about 11 and 11
+    // double-rate instructions (plus a few integer ones and one LDS read each) where the general library routines
+    // take 40 and 95.
+    // exp2: n = rint(256 x), r = x - n/256 (exact), 2^x = 2^(n>>8) * T[n&255] * 2^r, T[j] = 2^(j/256),
+    // 2^r - 1 = r (c1 + r (c2 + ... r c5)), c_k = ln(2)^k / k!, |r| <= 1/512 (remainder 1e-20).
+    // log2: x = 2^e * t, t in [1, 2), j = the top eight bits of t's fraction, u = t * R[j] - 1 in one fma with
+    // R[j] = 1/(1 + j/256) rounded, so 0 <= u < 2^-8 up to rounding and R[0] = 1 keeps t - 1 exact near 1;
+    // log2 t = G[j] + u (l1 + u (l2 + ... u l7)), G[j] = -log2 R[j] of the rounded R[j], l_k = (-1)^(k+1) / (k ln 2)
+    // (remainder 2e-18 relative). Both agree with the library to 1e-15 relative over their ranges (checked on
+    // the CPU against exp2/log2 of libm). The tables live in LDS, 6 KiB per block.
+    s << "#define SPN_DOUBLE_TABLES 1\n";
+    s << "__device__ const real_t spn_exp2_table[256] = {";
+    for (int j = 0; j < 256; ++j) s << (j ? ", " : "") << (j % 4 == 0 ? "\n  " : "") << e.lit(double(exp2l((long double)j / 256.0L)));
+    s << "};\n__device__ const real_t spn_log2_table[512] = {";
+    for (int j = 0; j < 256; ++j) {
+      const double recip = double(1.0L / (1.0L + (long double)j / 256.0L));
+      const double lg = j == 0 ? 0.0 : double(-log2l((long double)recip));
+      s << (j ? ", " : "") << (j % 2 == 0 ? "\n  " : "") << e.lit(recip) << ", " << e.lit(lg);
+    }
+    s << "};\n";
+    s << "#ifndef SPN_EXP2_TABLE\n__shared__ real_t spn_exp2_lds[256];\n__shared__ __attribute__((aligned(16))) real_t spn_log2_lds[512];\n"
+         "#define SPN_EXP2_TABLE spn_exp2_lds\n#define SPN_LOG2_TABLE spn_log2_lds\n#endif\n";
     s << "static __device__ " << mathAttr << " real_t spn_exp2(real_t x) {\n"
          "  x = x < -1100.0 ? -1100.0 : x;  // keeps NaN\n"
-         "  const real_t n = __builtin_rint(x), f = x - n;\n"
-         "  real_t p = 0x1.816193166d0f7p-40;\n"
-         "  p = __builtin_fma(p, f, 0x1.c3bd650fc2983p-36);\n  p = __builtin_fma(p, f, 0x1.e8cac7351bb22p-32);\n"
-         "  p = __builtin_fma(p, f, 0x1.e4cf5158b8ec7p-28);\n  p = __builtin_fma(p, f, 0x1.b5253d395e7c1p-24);\n"
-         "  p = __builtin_fma(p, f, 0x1.62c0223a5c822p-20);\n  p = __builtin_fma(p, f, 0x1.ffcbfc588b0c5p-17);\n"
-         "  p = __builtin_fma(p, f, 0x1.430912f86c786p-13);\n  p = __builtin_fma(p, f, 0x1.5d87fe78a6730p-10);\n"
-         "  p = __builtin_fma(p, f, 0x1.3b2ab6fba4e77p-7);\n  p = __builtin_fma(p, f, 0x1.c6b08d704a0bfp-5);\n"
-         "  p = __builtin_fma(p, f, 0x1.ebfbdff82c58ep-3);\n  p = __builtin_fma(p, f, 0x1.62e42fefa39efp-1);\n"
-         "  p = __builtin_fma(p, f, 1.0);\n"
-         "  return __builtin_ldexp(p, (int)n);\n}\n";
+         "  const real_t n = __builtin_rint(x * 256.0), r = __builtin_fma(n, -0x1p-8, x);\n"
+         "  const int ni = (int)n;\n"
+         "  const real_t t = SPN_EXP2_TABLE[ni & 255];\n"
+         "  real_t p = 0x1.5d87fe78a6731p-10;\n"
+         "  p = __builtin_fma(p, r, 0x1.3b2ab6fba4e77p-7);\n  p = __builtin_fma(p, r, 0x1.c6b08d704a0cp-5);\n"
+         "  p = __builtin_fma(p, r, 0x1.ebfbdff82c58fp-3);\n  p = __builtin_fma(p, r, 0x1.62e42fefa39efp-1);\n"
+         "  return __builtin_ldexp(__builtin_fma(t, p * r, t), ni >> 8);\n}\n";
     s << "static __device__ " << mathAttr << " real_t spn_log2(real_t x) {\n"
-         "  int e;\n  real_t t = __builtin_frexp(x, &e);\n"
-         "  const bool low = t < 0x1.6a09e667f3bcdp-1;\n  t = low ? t + t : t;\n  e = low ? e - 1 : e;\n"
-         "  const real_t z = (t - 1.0) / (t + 1.0), w = z * z;\n"
-         "  real_t p = 0x1.af286bca1af28p-5;\n"
-         "  p = __builtin_fma(p, w, 0x1.e1e1e1e1e1e1ep-5);\n  p = __builtin_fma(p, w, 0x1.1111111111111p-4);\n"
-         "  p = __builtin_fma(p, w, 0x1.3b13b13b13b14p-4);\n  p = __builtin_fma(p, w, 0x1.745d1745d1746p-4);\n"
-         "  p = __builtin_fma(p, w, 0x1.c71c71c71c71cp-4);\n  p = __builtin_fma(p, w, 0x1.2492492492492p-3);\n"
-         "  p = __builtin_fma(p, w, 0x1.999999999999ap-3);\n  p = __builtin_fma(p, w, 0x1.5555555555555p-2);\n"
-         "  p = __builtin_fma(p, w, 1.0);\n"
-         "  const real_t r = __builtin_fma(z * 0x1.71547652b82fep+1, p, (real_t)e);\n"
-         "  return x == 0.0 ? -__builtin_huge_val() : r;  // a sum whose terms are all impossible\n}\n";
+         "  union { real_t d; unsigned long long u; } c;\n  c.d = x;\n"
+         "  const unsigned hi = (unsigned)(c.u >> 32);\n"
+         "  const int e = (int)(hi >> 20) - 1023;\n"
+         "  const unsigned j = (hi >> 12) & 255u;\n"
+         "  c.u = (c.u & 0x000fffffffffffffull) | 0x3ff0000000000000ull;\n"
+         "  const real_t u = __builtin_fma(c.d, SPN_LOG2_TABLE[2 * j], -1.0);\n"
+         "  real_t p = 0x1.a61762a7aded9p-3;\n"
+         "  p = __builtin_fma(p, u, -0x1.ec709dc3a03fdp-3);\n  p = __builtin_fma(p, u, 0x1.2776c50ef9bfep-2);\n"
+         "  p = __builtin_fma(p, u, -0x1.71547652b82fep-2);\n  p = __builtin_fma(p, u, 0x1.ec709dc3a03fdp-2);\n"
+         "  p = __builtin_fma(p, u, -0x1.71547652b82fep-1);\n  p = __builtin_fma(p, u, 0x1.71547652b82fep+0);\n"
+         "  const real_t r = __builtin_fma(u, p, SPN_LOG2_TABLE[2 * j + 1] + (real_t)e);\n"
+         "  return x == 0.0 ? -__builtin_huge_val() : (x != x ? x : r);  // 0: a sum whose terms are all impossible\n}\n";
   }
   if (!e.log2Dom) {
     s << "static __device__ " << mathAttr << " real_t spn_exp(real_t x) { return " << (e.f64 ? "exp(x)" : "expf(x)") << "; }\n";
@@ -580,6 +595,10 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   if (minBlocks == 0 && js.tablesInLds && ldsTables > 40 * 1024 && ldsTables <= 80 * 1024 && tableFeatures <= 136) minBlocks = 2;
   s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK" << (minBlocks > 0 ? ", " + std::to_string(minBlocks) : std::string()) << ") " << js.entry
     << "(const feat_t* __restrict__ in, real_t* __restrict__ out, unsigned long long n) {\n";
+  if (e.log2Dom && e.f64)
+    s << "  for (unsigned t = threadIdx.x; t < 256; t += SPN_BLOCK) spn_exp2_lds[t] = spn_exp2_table[t];\n"
+         "  for (unsigned t = threadIdx.x; t < 512; t += SPN_BLOCK) spn_log2_lds[t] = spn_log2_table[t];\n"
+         "  __syncthreads();\n";
   if (js.tableEntries && js.tablesInLds) {
     s << "  __shared__ real_t tab[SPN_NTAB];\n"
          "  for (unsigned t = threadIdx.x; t < SPN_NTAB; t += SPN_BLOCK) tab[t] = spn_tables[t];\n"
