@@ -508,16 +508,23 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
       s << (j ? ", " : "") << (j % 2 == 0 ? "\n  " : "") << e.lit(recip) << ", " << e.lit(lg);
     }
     s << "};\n";
+    // The polynomial coefficients are read from LDS as well, once per kernel, and stay in registers: as literals
+    // every use costs two register moves, since a double constant cannot be an operand of the instruction itself.
+    // c5..c1 of exp2, then l7..l1 of log2.
+    s << "__device__ const real_t spn_poly[12] = {0x1.5d87fe78a6731p-10, 0x1.3b2ab6fba4e77p-7, 0x1.c6b08d704a0cp-5, 0x1.ebfbdff82c58fp-3, "
+         "0x1.62e42fefa39efp-1,\n  0x1.a61762a7aded9p-3, -0x1.ec709dc3a03fdp-3, 0x1.2776c50ef9bfep-2, -0x1.71547652b82fep-2, "
+         "0x1.ec709dc3a03fdp-2, -0x1.71547652b82fep-1, 0x1.71547652b82fep+0};\n";
     s << "#ifndef SPN_EXP2_TABLE\n__shared__ real_t spn_exp2_lds[256];\n__shared__ __attribute__((aligned(16))) real_t spn_log2_lds[512];\n"
-         "#define SPN_EXP2_TABLE spn_exp2_lds\n#define SPN_LOG2_TABLE spn_log2_lds\n#endif\n";
+         "__shared__ real_t spn_poly_lds[12];\n"
+         "#define SPN_EXP2_TABLE spn_exp2_lds\n#define SPN_LOG2_TABLE spn_log2_lds\n#define SPN_POLY spn_poly_lds\n#endif\n";
     s << "static __device__ " << mathAttr << " real_t spn_exp2(real_t x) {\n"
          "  x = x < -1100.0 ? -1100.0 : x;  // keeps NaN\n"
          "  const real_t n = __builtin_rint(x * 256.0), r = __builtin_fma(n, -0x1p-8, x);\n"
          "  const int ni = (int)n;\n"
          "  const real_t t = SPN_EXP2_TABLE[ni & 255];\n"
-         "  real_t p = 0x1.5d87fe78a6731p-10;\n"
-         "  p = __builtin_fma(p, r, 0x1.3b2ab6fba4e77p-7);\n  p = __builtin_fma(p, r, 0x1.c6b08d704a0cp-5);\n"
-         "  p = __builtin_fma(p, r, 0x1.ebfbdff82c58fp-3);\n  p = __builtin_fma(p, r, 0x1.62e42fefa39efp-1);\n"
+         "  real_t p = SPN_POLY[0];\n"
+         "  p = __builtin_fma(p, r, SPN_POLY[1]);\n  p = __builtin_fma(p, r, SPN_POLY[2]);\n"
+         "  p = __builtin_fma(p, r, SPN_POLY[3]);\n  p = __builtin_fma(p, r, SPN_POLY[4]);\n"
          "  return __builtin_ldexp(__builtin_fma(t, p * r, t), ni >> 8);\n}\n";
     s << "static __device__ " << mathAttr << " real_t spn_log2(real_t x) {\n"
          "  union { real_t d; unsigned long long u; } c;\n  c.d = x;\n"
@@ -526,10 +533,10 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
          "  const unsigned j = (hi >> 12) & 255u;\n"
          "  c.u = (c.u & 0x000fffffffffffffull) | 0x3ff0000000000000ull;\n"
          "  const real_t u = __builtin_fma(c.d, SPN_LOG2_TABLE[2 * j], -1.0);\n"
-         "  real_t p = 0x1.a61762a7aded9p-3;\n"
-         "  p = __builtin_fma(p, u, -0x1.ec709dc3a03fdp-3);\n  p = __builtin_fma(p, u, 0x1.2776c50ef9bfep-2);\n"
-         "  p = __builtin_fma(p, u, -0x1.71547652b82fep-2);\n  p = __builtin_fma(p, u, 0x1.ec709dc3a03fdp-2);\n"
-         "  p = __builtin_fma(p, u, -0x1.71547652b82fep-1);\n  p = __builtin_fma(p, u, 0x1.71547652b82fep+0);\n"
+         "  real_t p = SPN_POLY[5];\n"
+         "  p = __builtin_fma(p, u, SPN_POLY[6]);\n  p = __builtin_fma(p, u, SPN_POLY[7]);\n"
+         "  p = __builtin_fma(p, u, SPN_POLY[8]);\n  p = __builtin_fma(p, u, SPN_POLY[9]);\n"
+         "  p = __builtin_fma(p, u, SPN_POLY[10]);\n  p = __builtin_fma(p, u, SPN_POLY[11]);\n"
          "  const real_t r = __builtin_fma(u, p, SPN_LOG2_TABLE[2 * j + 1] + (real_t)e);\n"
          "  return x == 0.0 ? -__builtin_huge_val() : (x != x ? x : r);  // 0: a sum whose terms are all impossible\n}\n";
   }
@@ -598,6 +605,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   if (e.log2Dom && e.f64)
     s << "  for (unsigned t = threadIdx.x; t < 256; t += SPN_BLOCK) spn_exp2_lds[t] = spn_exp2_table[t];\n"
          "  for (unsigned t = threadIdx.x; t < 512; t += SPN_BLOCK) spn_log2_lds[t] = spn_log2_table[t];\n"
+         "  if (threadIdx.x < 12) spn_poly_lds[threadIdx.x] = spn_poly[threadIdx.x];\n"
          "  __syncthreads();\n";
   if (js.tableEntries && js.tablesInLds) {
     s << "  __shared__ real_t tab[SPN_NTAB];\n"

@@ -16,8 +16,8 @@ def _routines(native, tmp_path):
     src = k.source()
     os.remove(k.fileName())
     assert src.count("spn_exp2(") > 200 and src.count("spn_log2(") > 70 and "spn_exp(" not in src and "spn_log(" not in src
-    parts = ["#define SPN_EXP2_TABLE spn_exp2_table\n#define SPN_LOG2_TABLE spn_log2_table\n"]
-    for name in ("spn_exp2_table", "spn_log2_table"):   # the kernel copies these into LDS; on the CPU they are read where they are
+    parts = ["#define SPN_EXP2_TABLE spn_exp2_table\n#define SPN_LOG2_TABLE spn_log2_table\n#define SPN_POLY spn_poly\n"]
+    for name in ("spn_exp2_table", "spn_log2_table", "spn_poly"):   # the kernel copies these into LDS; on the CPU they are read where they are
         m = re.search(r"__device__ const real_t " + name + r"\[\d+\] = \{.*?\};\n", src, re.S)
         assert m, name
         parts.append(m.group(0).replace("__device__ ", "static "))
