@@ -491,16 +491,17 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     // rounding, logarithms of sums in [1, fan-in] or of exactly 0), by table and short polynomial: about 11 and 11
     // double-rate instructions (plus a few integer ones and one LDS read each) where the general library routines
     // take 40 and 95.
-    // exp2: n = rint(256 x), r = x - n/256 (exact), 2^x = 2^(n>>8) * T[n&255] * 2^r, T[j] = 2^(j/256),
-    // 2^r - 1 = r (c1 + r (c2 + ... r c5)), c_k = ln(2)^k / k!, |r| <= 1/512 (remainder 1e-20).
+    // exp2: n = rint(64 x), r = x - n/64 (exact), 2^x = 2^(n>>6) * T[n&63] * 2^r, T[j] = 2^(j/64),
+    // 2^r - 1 = r (c1 + r (c2 + ... r c5)), c_k = ln(2)^k / k!, |r| <= 1/128 (remainder 4e-17;
+    // a table of 256 entries has its reads spread over sixteen times the width of the LDS banks, this one over four).
     // log2: x = 2^e * t, t in [1, 2), j = the top eight bits of t's fraction, u = t * R[j] - 1 in one fma with
     // R[j] = 1/(1 + j/256) rounded, so 0 <= u < 2^-8 up to rounding and R[0] = 1 keeps t - 1 exact near 1;
     // log2 t = G[j] + u (l1 + u (l2 + ... u l7)), G[j] = -log2 R[j] of the rounded R[j], l_k = (-1)^(k+1) / (k ln 2)
     // (remainder 2e-18 relative). Both agree with the library to 1e-15 relative over their ranges (checked on
-    // the CPU against exp2/log2 of libm). The tables live in LDS, 6 KiB per block.
+    // the CPU against exp2/log2 of libm). The tables live in LDS, 4.5 KiB per block.
     s << "#define SPN_DOUBLE_TABLES 1\n";
-    s << "__device__ const real_t spn_exp2_table[256] = {";
-    for (int j = 0; j < 256; ++j) s << (j ? ", " : "") << (j % 4 == 0 ? "\n  " : "") << e.lit(double(exp2l((long double)j / 256.0L)));
+    s << "__device__ const real_t spn_exp2_table[64] = {";
+    for (int j = 0; j < 64; ++j) s << (j ? ", " : "") << (j % 4 == 0 ? "\n  " : "") << e.lit(double(exp2l((long double)j / 64.0L)));
     s << "};\n__device__ const real_t spn_log2_table[512] = {";
     for (int j = 0; j < 256; ++j) {
       const double recip = double(1.0L / (1.0L + (long double)j / 256.0L));
@@ -514,18 +515,18 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     s << "__device__ const real_t spn_poly[12] = {0x1.5d87fe78a6731p-10, 0x1.3b2ab6fba4e77p-7, 0x1.c6b08d704a0cp-5, 0x1.ebfbdff82c58fp-3, "
          "0x1.62e42fefa39efp-1,\n  0x1.a61762a7aded9p-3, -0x1.ec709dc3a03fdp-3, 0x1.2776c50ef9bfep-2, -0x1.71547652b82fep-2, "
          "0x1.ec709dc3a03fdp-2, -0x1.71547652b82fep-1, 0x1.71547652b82fep+0};\n";
-    s << "#ifndef SPN_EXP2_TABLE\n__shared__ real_t spn_exp2_lds[256];\n__shared__ __attribute__((aligned(16))) real_t spn_log2_lds[512];\n"
+    s << "#ifndef SPN_EXP2_TABLE\n__shared__ real_t spn_exp2_lds[64];\n__shared__ __attribute__((aligned(16))) real_t spn_log2_lds[512];\n"
          "__shared__ real_t spn_poly_lds[12];\n"
          "#define SPN_EXP2_TABLE spn_exp2_lds\n#define SPN_LOG2_TABLE spn_log2_lds\n#define SPN_POLY spn_poly_lds\n#endif\n";
     s << "static __device__ " << mathAttr << " real_t spn_exp2(real_t x) {\n"
          "  x = x < -1100.0 ? -1100.0 : x;  // keeps NaN\n"
-         "  const real_t n = __builtin_rint(x * 256.0), r = __builtin_fma(n, -0x1p-8, x);\n"
+         "  const real_t n = __builtin_rint(x * 64.0), r = __builtin_fma(n, -0x1p-6, x);\n"
          "  const int ni = (int)n;\n"
-         "  const real_t t = SPN_EXP2_TABLE[ni & 255];\n"
+         "  const real_t t = SPN_EXP2_TABLE[ni & 63];\n"
          "  real_t p = SPN_POLY[0];\n"
          "  p = __builtin_fma(p, r, SPN_POLY[1]);\n  p = __builtin_fma(p, r, SPN_POLY[2]);\n"
          "  p = __builtin_fma(p, r, SPN_POLY[3]);\n  p = __builtin_fma(p, r, SPN_POLY[4]);\n"
-         "  return __builtin_ldexp(__builtin_fma(t, p * r, t), ni >> 8);\n}\n";
+         "  return __builtin_ldexp(__builtin_fma(t, p * r, t), ni >> 6);\n}\n";
     s << "static __device__ " << mathAttr << " real_t spn_log2(real_t x) {\n"
          "  union { real_t d; unsigned long long u; } c;\n  c.d = x;\n"
          "  const unsigned hi = (unsigned)(c.u >> 32);\n"
@@ -603,7 +604,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK" << (minBlocks > 0 ? ", " + std::to_string(minBlocks) : std::string()) << ") " << js.entry
     << "(const feat_t* __restrict__ in, real_t* __restrict__ out, unsigned long long n) {\n";
   if (e.log2Dom && e.f64)
-    s << "  for (unsigned t = threadIdx.x; t < 256; t += SPN_BLOCK) spn_exp2_lds[t] = spn_exp2_table[t];\n"
+    s << "  for (unsigned t = threadIdx.x; t < 64; t += SPN_BLOCK) spn_exp2_lds[t] = spn_exp2_table[t];\n"
          "  for (unsigned t = threadIdx.x; t < 512; t += SPN_BLOCK) spn_log2_lds[t] = spn_log2_table[t];\n"
          "  if (threadIdx.x < 12) spn_poly_lds[threadIdx.x] = spn_poly[threadIdx.x];\n"
          "  __syncthreads();\n";
