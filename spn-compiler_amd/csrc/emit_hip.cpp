@@ -23,6 +23,25 @@ struct Emitter {
   std::vector<double> tablePool;
   std::vector<uint32_t> tableOffset;   // per node (for a paired leaf: offset of the joint table, held by the first of the pair)
   std::vector<uint32_t> partner;       // per node: the table leaf it shares a joint table with, or UINT32_MAX
+  // Tables read with the same index (all leaves on one feature, all joint tables over one pair of features) are
+  // interleaved in groups of four or two: entry i of the group holds the members' values for index i side by side,
+  // and one 16- or 8-byte read fetches them all.
+  struct TableGroup {
+    uint32_t offset = 0, width = 1;      // pool offset in entries of the first member; members side by side per entry
+    uint32_t stride = 1;                 // entries from one index value to the next: 4 in a block of four columns
+    uint32_t fa = 0, fb = UINT32_MAX;    // index: t_fa, or t_fa * rowLen(fb) + t_fb for joint tables
+    std::vector<uint32_t> members;       // table leaves (for a joint table: the first leaf of the pair), in node order
+    bool loaded = false;
+  };
+  std::vector<TableGroup> groups;
+  std::vector<uint32_t> groupOf, laneOf;  // per node (first leaf of a pair): its group and its position in the group's entries
+  std::unordered_map<uint64_t, bool> jointIndexNamed;  // pairs of features whose joint index has been emitted
+  std::vector<uint64_t> keyOrder;                                   // indices in order of first appearance
+  std::unordered_map<uint64_t, std::vector<uint32_t>> unitsByKey;  // tables (joint tables: first leaf) per index
+  bool packedIndices = false;                                       // blocks of four columns: byte offsets of the entries, four features to a register
+  unsigned extractions = 0;                                         // numbers the statements that take a byte offset out of its register
+  bool recording = false;                                           // first pass: only the order of table uses matters
+  std::vector<uint32_t> useOrder, useRank;                          // tables in order of use; per table: its place in that order
   std::vector<uint32_t> featTableLen;  // per feature: longest table of any leaf on it (0 = none)
   std::vector<bool> featGauss;         // per feature: used by a Gaussian leaf
   std::vector<bool> featUsed;
@@ -101,17 +120,6 @@ struct Emitter {
     tableOffset.assign(g.nodes.size(), 0);
     partner.assign(g.nodes.size(), UINT32_MAX);
     auto isTable = [&](uint32_t c) { return g.nodes[c].kind == NodeKind::Categorical || g.nodes[c].kind == NodeKind::Histogram; };
-    auto padded = [&](uint32_t c) {
-      const auto& n = g.nodes[c];
-      const uint32_t L = featTableLen[n.feature];
-      std::vector<double> t;
-      for (uint32_t j = 0; j <= L; ++j) {
-        double p = j < n.table.size() ? n.table[j] : 0.0;
-        t.push_back(logSpace ? logConst(p) : p);
-      }
-      if (g.supportMarginal) t.push_back(logSpace ? 0.0 : 1.0);
-      return t;
-    };
     auto rowLen = [&](uint32_t feature) { return size_t(featTableLen[feature]) + (g.supportMarginal ? 2 : 1); };
     // Joint tables: two table leaves read only by the same product are replaced by one table over
     // the pair of indices, J[i][j] = T_a[i] (+ or *) T_b[j], combined in double. One LDS read and one
@@ -148,19 +156,212 @@ struct Emitter {
       partner[c.a] = c.b;
       partner[c.b] = c.a;
     }
+    // Units (single tables and joint tables) by index, in node order.
     for (uint32_t i = 0; i < g.nodes.size(); ++i) {
       if (!isTable(i)) continue;
       if (partner[i] != UINT32_MAX && partner[i] < i) continue;  // second leaf of a pair: lives in the joint table
-      tableOffset[i] = uint32_t(tablePool.size());
-      std::vector<double> a = padded(i);
-      if (partner[i] == UINT32_MAX) {
-        tablePool.insert(tablePool.end(), a.begin(), a.end());
-      } else {
-        std::vector<double> b = padded(partner[i]);
-        for (double x : a)
-          for (double y : b) tablePool.push_back(logSpace ? x + y : x * y);
-      }
+      const uint64_t fb = partner[i] == UINT32_MAX ? 0 : uint64_t(g.nodes[partner[i]].feature) + 1;
+      const uint64_t key = o.groupedTables ? (uint64_t(g.nodes[i].feature) << 32) | fb : uint64_t(i);  // ungrouped: every table on its own
+      if (!unitsByKey.count(key)) keyOrder.push_back(key);
+      unitsByKey[key].push_back(i);
     }
+    useRank.assign(g.nodes.size(), 0);
+    if (o.groupedTables && !unitsByKey.empty()) recordUseOrder();
+    buildPool();
+  }
+
+  std::vector<double> unitValues(uint32_t i) const {
+    auto padded = [&](uint32_t c) {
+      const auto& n = g.nodes[c];
+      const uint32_t L = featTableLen[n.feature];
+      std::vector<double> t;
+      for (uint32_t j = 0; j <= L; ++j) {
+        double p = j < n.table.size() ? n.table[j] : 0.0;
+        t.push_back(logSpace ? logConst(p) : p);
+      }
+      if (g.supportMarginal) t.push_back(logSpace ? 0.0 : 1.0);
+      return t;
+    };
+    std::vector<double> a = padded(i);
+    if (partner[i] == UINT32_MAX) return a;
+    std::vector<double> b = padded(partner[i]), joint;
+    for (double x : a)
+      for (double y : b) joint.push_back(logSpace ? x + y : x * y);
+    return joint;
+  }
+
+  // Groups of four, two and one over the units of every index, in the order the lists hold them, and the pool.
+  void buildPool() {
+    const size_t realBytes = f64 ? 8 : 4, limit = (size_t(o.tableBudgetKiB) + size_t(o.tablePadKiB)) * 1024;
+    bool shared = false;
+    for (const auto& kv : unitsByKey) shared = shared || kv.second.size() > 1;
+    // Blocks of four columns go with packed indices: the byte offset of a feature's entry, index * 4 * sizeof(real_t),
+    // must fit into eight bits, and the indices must all be at hand when the kernel body starts.
+    for (uint32_t f = 0; f < g.numFeatures; ++f)
+      if (featTableLen[f] && (featTableLen[f] + (g.supportMarginal ? 1u : 0u)) * 4 * realBytes > 255) shared = false;
+    if (!vectorRows || !o.eagerIndices) shared = false;
+    size_t reads = 0;
+    for (const auto& kv : unitsByKey) reads += kv.second.size();
+    if (reads < size_t(o.tableGroupMinReads)) shared = false;  // too few reads for the LDS to matter
+    packedIndices = false;
+    for (int attempt = shared ? 0 : 1; attempt < 2; ++attempt) {
+      const bool blocks = attempt == 0;  // else every table on its own, entries side by side
+      groups.clear();
+      tablePool.clear();
+      groupOf.assign(g.nodes.size(), UINT32_MAX);
+      laneOf.assign(g.nodes.size(), 0);
+      for (uint64_t key : keyOrder) {
+        const std::vector<uint32_t>& list = unitsByKey[key];
+        const size_t rows = unitValues(list[0]).size(), firstGroup = groups.size();
+        for (size_t pos = 0; pos < list.size();) {
+          size_t count = 1;
+          while (blocks && count < 4 && pos + count < list.size() &&
+                 useRank[list[pos + count]] - useRank[list[pos]] <= uint32_t(o.tableGroupWindow))
+            ++count;
+          TableGroup G;
+          G.width = uint32_t(count);
+          G.stride = blocks ? 4 : 1;
+          G.fa = g.nodes[list[pos]].feature;
+          G.fb = partner[list[pos]] == UINT32_MAX ? UINT32_MAX : g.nodes[partner[list[pos]]].feature;
+          for (size_t k = 0; k < count; ++k) {
+            groupOf[list[pos + k]] = uint32_t(groups.size());
+            laneOf[list[pos + k]] = uint32_t(k);
+            G.members.push_back(list[pos + k]);
+          }
+          groups.push_back(G);
+          pos += count;
+        }
+        // Columns: groups of four and three open a block of their own, pairs take a half, single tables whatever
+        // is free (the fourth column beside three tables first).
+        const size_t base = tablePool.size();
+        std::vector<uint32_t> freeColumns;  // per block of this index: bit c set = column c is free
+        auto place = [&](TableGroup& G, size_t block, uint32_t column) {
+          if (block == freeColumns.size()) {
+            freeColumns.push_back(0xfu);
+            tablePool.resize(tablePool.size() + rows * G.stride, 0.0);
+          }
+          for (uint32_t c = 0; c < G.width; ++c) freeColumns[block] &= ~(1u << (column + c));
+          G.offset = uint32_t(base + block * rows * G.stride + column);
+          for (size_t m = 0; m < G.members.size(); ++m) {
+            const std::vector<double> col = unitValues(G.members[m]);
+            for (size_t r = 0; r < rows; ++r) tablePool[G.offset + r * G.stride + m] = col[r];
+            tableOffset[G.members[m]] = G.offset;
+          }
+        };
+        for (uint32_t width : {4u, 3u, 2u, 1u}) {
+          for (size_t k = firstGroup; k < groups.size(); ++k) {
+            TableGroup& G = groups[k];
+            if (G.width != width) continue;
+            if (!blocks) {
+              G.offset = uint32_t(tablePool.size());
+              tablePool.resize(tablePool.size() + rows, 0.0);
+              const std::vector<double> col = unitValues(G.members[0]);
+              std::copy(col.begin(), col.end(), tablePool.begin() + G.offset);
+              tableOffset[G.members[0]] = G.offset;
+              continue;
+            }
+            size_t block = freeColumns.size();
+            uint32_t column = 0;
+            for (size_t q = 0; q < freeColumns.size() && block == freeColumns.size() && width <= 2; ++q) {
+              if (width == 2 && (freeColumns[q] & 0xcu) == 0xcu) block = q, column = 2;
+              for (uint32_t c = 4; c-- > 0 && width == 1;)
+                if (freeColumns[q] & (1u << c)) block = q, column = c;
+            }
+            place(G, block, column);
+          }
+        }
+      }
+      if (blocks && tablePool.size() * realBytes <= limit) packedIndices = true;
+      if (!blocks || packedIndices) break;  // blocks that outgrow the LDS share: plain tables
+    }
+  }
+
+  // A group's vector stays in registers from its read, at the first member's use, to the last member's use. The
+  // members of a group are therefore tables of its index that the kernel needs shortly after one another (the
+  // children of one sum, as a rule): a first pass over the graph records the order in which the tables are used.
+  void recordUseOrder() {
+    recording = true;
+    emitNode(g.root());
+    recording = false;
+    useRank.assign(g.nodes.size(), UINT32_MAX);
+    for (size_t k = 0; k < useOrder.size(); ++k)
+      if (useRank[useOrder[k]] == UINT32_MAX) useRank[useOrder[k]] = uint32_t(k);
+    for (auto& kv : unitsByKey)
+      std::stable_sort(kv.second.begin(), kv.second.end(), [&](uint32_t x, uint32_t y) { return useRank[x] < useRank[y]; });
+    body.str("");
+    body.clear();
+    std::fill(emitted.begin(), emitted.end(), false);
+    std::fill(featPrepared.begin(), featPrepared.end(), false);
+    foldedWeight.clear();
+    jointIndexNamed.clear();
+    useOrder.clear();
+  }
+
+  // Packed indices: register P<k> holds, for features 4k .. 4k+3, the byte offset of the feature's entry within a
+  // block of four columns (index * 4 * sizeof(real_t)), eight bits each. An offset is taken out where a group is
+  // read, by a statement of its own every time (the number in its comment keeps the compiler from merging them):
+  // merged, a hundred offsets would stay in registers for the whole kernel, which is what the packing is there
+  // to avoid.
+  void emitPackedIndices() {
+    const unsigned entryBytes = 4 * (f64 ? 8 : 4);
+    for (uint32_t k = 0; k * 4 < g.numFeatures; ++k) {
+      std::string expr;
+      for (uint32_t j = 0; j < 4 && k * 4 + j < g.numFeatures; ++j) {
+        const uint32_t f = k * 4 + j;
+        if (!featUsed[f] || !featTableLen[f]) continue;
+        expr += (expr.empty() ? "" : " | ") + std::string("((t") + std::to_string(f) + " * " + std::to_string(entryBytes) + "u) << " + std::to_string(8 * j) + ")";
+      }
+      if (!expr.empty()) body << "  const unsigned P" << k << " = " << expr << ";\n";
+    }
+  }
+  std::string byteOffset(uint32_t f) {
+    const std::string name = "b" + std::to_string(extractions);
+    body << "  unsigned " << name << ";\n  asm(\"v_bfe_u32 %0, %1, " << 8 * (f % 4) << ", 8 ; " << extractions << "\" : \"=v\"(" << name << ") : \"v\"(P" << f / 4 << "));\n";
+    ++extractions;
+    return name;
+  }
+
+  // The index expression of a group: the clamped feature index, or the named joint index of its two features
+  // (packed indices: the byte offset of the entry).
+  std::string groupIndex(const TableGroup& G) {
+    if (packedIndices) {
+      const std::string a = byteOffset(G.fa);
+      if (G.fb == UINT32_MAX) return a;
+      const std::string b = byteOffset(G.fb);
+      return "(" + a + " * " + std::to_string(featTableLen[G.fb] + (g.supportMarginal ? 2 : 1)) + "u + " + b + ")";
+    }
+    if (G.fb == UINT32_MAX) return "t" + std::to_string(G.fa);
+    const std::string name = "k" + std::to_string(G.fa) + "_" + std::to_string(G.fb);
+    const uint64_t key = (uint64_t(G.fa) << 32) | G.fb;
+    if (!jointIndexNamed[key]) {
+      jointIndexNamed[key] = true;
+      body << "  const unsigned " << name << " = t" << G.fa << " * " << (featTableLen[G.fb] + (g.supportMarginal ? 2 : 1)) << "u + t" << G.fb << ";\n";
+    }
+    return name;
+  }
+
+  // The value of table unit i (a table leaf, or the first leaf of a pair): a plain read for a table on its own,
+  // else a component of its group's vector, which is read where its first member is needed.
+  std::string tableValue(uint32_t i) {
+    if (recording) {
+      useOrder.push_back(i);
+      return "0";
+    }
+    TableGroup& G = groups[groupOf[i]];
+    if (packedIndices) {
+      const std::string q = "q" + std::to_string(groupOf[i]);
+      if (!G.loaded) {
+        G.loaded = true;
+        const std::string idx = groupIndex(G);
+        const char* type = G.width == 1 ? "real_t" : (G.width == 2 ? "spn_r2" : "spn_r4");  // three tables: the fourth column comes along unused
+        body << "  const " << type << " " << q << " = *reinterpret_cast<const " << type << "*>(reinterpret_cast<const char*>(tab + " << G.offset
+             << "u) + " << idx << ");\n";
+      }
+      return G.width == 1 ? q : q + "[" + std::to_string(laneOf[i]) + "]";
+    }
+    if (G.fb == UINT32_MAX) return "tab[" + std::to_string(G.offset) + "u + t" + std::to_string(G.fa) + "]";
+    return "tab[" + std::to_string(G.offset) + "u + t" + std::to_string(G.fa) + " * " +
+           std::to_string(featTableLen[G.fb] + (g.supportMarginal ? 2 : 1)) + "u + t" + std::to_string(G.fb) + "]";
   }
 
   // Emitted right before the first leaf that reads feature f, so that for wide rows the load
@@ -242,8 +443,8 @@ struct Emitter {
       emitFeaturePrep(fb);
       emitted[a] = emitted[b] = true;
       const std::string name = "j" + std::to_string(a);
-      body << "  const real_t " << name << " = tab[" << tableOffset[a] << "u + t" << fa << " * " << (featTableLen[fb] + (g.supportMarginal ? 2 : 1))
-           << "u + t" << fb << "];\n";
+      const std::string value = tableValue(a);  // may emit the read of the group
+      body << "  const real_t " << name << " = " << value << ";\n";
       ops.push_back(name);
     }
     return ops;
@@ -319,8 +520,11 @@ struct Emitter {
       }
       case NodeKind::Categorical:
       case NodeKind::Histogram:
-        body << "  const real_t " << v(i) << " = tab[" << tableOffset[i] << "u + t" << n.feature << "];\n";
+      {
+        const std::string value = tableValue(i);  // may emit the read of the group
+        body << "  const real_t " << v(i) << " = " << value << ";\n";
         break;
+      }
       case NodeKind::Product: {
         if (logSpace && fusableProduct(i)) {
           emitFusedProduct(i);
@@ -428,10 +632,17 @@ unsigned pickVectorBytes(unsigned rowBytes, unsigned elemBytes) {
 
 JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   Emitter e(g, o);
+  // Short rows are fetched with the widest vector loads their size allows, all samples of a
+  // lane up front; wide rows are read feature by feature next to the first use.
+  e.vectorRows = g.numFeatures * g.ftype.bytes <= 512;
   e.prepare();
   JitSource js;
   js.entry = "spn_kernel";
   js.blockSize = o.blockSize ? unsigned(o.blockSize) : 256u;
+  // Grouped tables with packed indices leave the kernel at about 140 registers and take up to 80 KiB of LDS: one
+  // block of 1024 threads per CU then runs four waves per SIMD on one copy of the tables (C3: 1.19 ms with two
+  // blocks of 256, 1.18 ms with two of 512, 1.06 ms with one of 1024).
+  if (o.blockSize == 0 && e.packedIndices) js.blockSize = 1024;
   js.bytesPerResult = e.f64 ? 8 : 4;
   js.tableEntries = unsigned(e.tablePool.size());
   const unsigned realBytes = e.f64 ? 8 : 4;
@@ -441,9 +652,15 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   const unsigned F = g.numFeatures;
   const unsigned eb = g.ftype.bytes;
   const unsigned rowBytes = F * eb;
-  // Short rows are fetched with the widest vector loads their size allows, all samples of a
-  // lane up front; wide rows are read feature by feature next to the first use.
-  e.vectorRows = rowBytes <= 512;
+  // Rows held in registers: the clamped table indices are derived right away, so that a raw feature
+  // value and its index are never live together for long.
+  auto emitBody = [&] {
+    if (e.vectorRows && o.eagerIndices)
+      for (uint32_t f = 0; f < F; ++f)
+        if (e.featUsed[f] && e.featTableLen[f]) e.emitFeaturePrep(f);
+    if (e.packedIndices) e.emitPackedIndices();
+    e.emitNode(g.root());
+  };
   const unsigned vb = e.vectorRows ? pickVectorBytes(rowBytes, eb) : eb;
   const unsigned vw = vb / eb;
   js.inputAlign = vb;
@@ -479,7 +696,8 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   s << "#define SPN_F " << F << "\n#define SPN_BLOCK " << js.blockSize << "\n#define SPN_U " << U << "\n";
   if (js.tableEntries) {
     s << "#define SPN_NTAB " << js.tableEntries << "\n";
-    s << "__device__ const real_t spn_tables[SPN_NTAB] = {";
+    s << "typedef real_t spn_r2 __attribute__((ext_vector_type(2)));\ntypedef real_t spn_r4 __attribute__((ext_vector_type(4)));\n";
+    s << "__device__ __attribute__((aligned(32))) const real_t spn_tables[SPN_NTAB] = {";
     for (size_t i = 0; i < e.tablePool.size(); ++i) s << (i ? ", " : "") << (i % 8 == 0 ? "\n  " : "") << e.lit(e.tablePool[i]);
     s << "};\n";
   }
@@ -575,12 +793,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     s << "}\n";
   }
 
-  // Rows held in registers: derive the clamped table indices right away, so that a raw feature
-  // value and its index are never live together for long.
-  if (e.vectorRows && o.eagerIndices)
-    for (uint32_t f = 0; f < F; ++f)
-      if (e.featUsed[f] && e.featTableLen[f]) e.emitFeaturePrep(f);
-  e.emitNode(g.root());
+  emitBody();
   if (e.vectorRows)
     s << "static __device__ __forceinline__ real_t spn_eval(const feat_t (&x)[SPN_F], const real_t* __restrict__ tab) {\n";
   else
@@ -600,6 +813,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   unsigned tableFeatures = 0;
   for (uint32_t f = 0; f < F; ++f) tableFeatures += e.featTableLen[f] ? 1 : 0;
   int minBlocks = o.minBlocksPerCU;
+  if (minBlocks == 0 && js.blockSize == 1024) minBlocks = 1;
   if (minBlocks == 0 && js.tablesInLds && ldsTables > 40 * 1024 && ldsTables <= 80 * 1024 && tableFeatures <= 136) minBlocks = 2;
   s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK" << (minBlocks > 0 ? ", " + std::to_string(minBlocks) : std::string()) << ") " << js.entry
     << "(const feat_t* __restrict__ in, real_t* __restrict__ out, unsigned long long n) {\n";
@@ -609,7 +823,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
          "  if (threadIdx.x < 12) spn_poly_lds[threadIdx.x] = spn_poly[threadIdx.x];\n"
          "  __syncthreads();\n";
   if (js.tableEntries && js.tablesInLds) {
-    s << "  __shared__ real_t tab[SPN_NTAB];\n"
+    s << "  __shared__ __attribute__((aligned(32))) real_t tab[SPN_NTAB];\n"
          "  for (unsigned t = threadIdx.x; t < SPN_NTAB; t += SPN_BLOCK) tab[t] = spn_tables[t];\n"
          "  __syncthreads();\n";
   } else if (js.tableEntries) {

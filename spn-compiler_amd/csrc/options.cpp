@@ -98,6 +98,17 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       o.eagerIndices = parseBool(val);
     } else if (key == "hip-joint-tables") {
       o.jointTables = parseBool(val);
+    } else if (key == "hip-grouped-tables") {
+      o.groupedTables = parseBool(val);
+    } else if (key == "hip-table-group-min-reads") {
+      o.tableGroupMinReads = parseInt(key, val);
+      if (o.tableGroupMinReads < 0) throw std::runtime_error("hip-table-group-min-reads must not be negative");
+    } else if (key == "hip-table-group-window") {
+      o.tableGroupWindow = parseInt(key, val);
+      if (o.tableGroupWindow < 0) throw std::runtime_error("hip-table-group-window must not be negative");
+    } else if (key == "hip-table-pad-kib") {
+      o.tablePadKiB = parseInt(key, val);
+      if (o.tablePadKiB < 0 || o.tablePadKiB > 64) throw std::runtime_error("hip-table-pad-kib must be in [0,64]");
     } else if (key == "hip-interp-short-slots") {
       o.interpShortSlots = parseInt(key, val);
       if (o.interpShortSlots < 0 || o.interpShortSlots > 160) throw std::runtime_error("hip-interp-short-slots must be in [0,160]");
@@ -118,7 +129,7 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       o.inlineMath = val == "auto" ? -1 : (parseBool(val) ? 1 : 0);
     } else if (key == "hip-table-budget-kib") {
       o.tableBudgetKiB = parseInt(key, val);
-      if (o.tableBudgetKiB < 0 || o.tableBudgetKiB > 62) throw std::runtime_error("hip-table-budget-kib must be in [0,62]");
+      if (o.tableBudgetKiB < 0 || o.tableBudgetKiB > 140) throw std::runtime_error("hip-table-budget-kib must be in [0,140]");
     } else if (key == "hip-joint-max-entries") {
       o.jointMaxEntries = parseInt(key, val);
       if (o.jointMaxEntries < 0 || o.jointMaxEntries > 4096) throw std::runtime_error("hip-joint-max-entries must be in [0,4096]");
@@ -130,8 +141,8 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       if (o.blocksPerCU < -1 || o.blocksPerCU > 64) throw std::runtime_error("hip-blocks-per-cu must be in [-1,64]");
     } else if (key == "hip-block-size") {
       o.blockSize = parseInt(key, val);
-      if (o.blockSize != 0 && o.blockSize != 64 && o.blockSize != 128 && o.blockSize != 256 && o.blockSize != 512)
-        throw std::runtime_error("hip-block-size must be 64, 128, 256 or 512");
+      if (o.blockSize != 0 && o.blockSize != 64 && o.blockSize != 128 && o.blockSize != 256 && o.blockSize != 512 && o.blockSize != 1024)
+        throw std::runtime_error("hip-block-size must be 64, 128, 256, 512 or 1024");
     } else if (ignoredKeys().count(key)) {
       // accepted for compatibility, no effect on the HIP target
     } else {

@@ -36,6 +36,10 @@ struct CompileOptions {
   bool jointTables = true;                     // "hip-joint-tables": pair table leaves of a product into joint tables
   int machineLicm = -1;                        // "hip-machine-licm": machine LICM for generated kernels on (1), off (0) or decided per kernel (-1)
   int inlineMath = -1;                         // "hip-inline-math": exp/log routines inlined (1), called (0) or decided by graph size (-1)
+  bool groupedTables = true;                   // "hip-grouped-tables": tables read with the same index are interleaved in blocks of four columns and fetched up to four per read
+  int tableGroupMinReads = 200;                // "hip-table-group-min-reads": graphs with fewer table reads per sample keep plain tables
+  int tableGroupWindow = 96;                   // "hip-table-group-window": tables of a group are used within this many table uses of each other
+  int tablePadKiB = 18;                        // "hip-table-pad-kib": LDS beyond the table budget that blocks of four columns may take (unused columns)
   int tableBudgetKiB = 62;                     // "hip-table-budget-kib": LDS the table pool may grow to when leaves are paired into joint tables
   int jointMaxEntries = 160;                   // "hip-joint-max-entries": largest joint table (entries) a pair of table leaves may get
   int interpShortSlots = 0;                    // "hip-interp-short-slots": LDS value slots per lane the interpreter program aims for (0 = automatic)

@@ -146,6 +146,72 @@ def test_benchmark_configurations(native, cfg, variant):
     assert np.abs(got - c_oracle.ll_f32(m, X, marginal=c["marginal"])).max() <= F32_TOL
 
 
+GROUPED = {
+    "default": {},                                        # blocks of four columns, packed indices, one block of 1024 threads
+    "plain": {"hip-grouped-tables": "false"},
+    "singles": {"hip-table-group-window": 0},             # blocks of four columns, every table read on its own
+    "wide-window": {"hip-table-group-window": 1000},
+    "no-room": {"hip-table-pad-kib": 0},                  # blocks do not fit: plain tables
+    "no-joint": {"hip-joint-tables": "false"},
+    "small-pool": {"hip-table-budget-kib": 30},           # no pairing, and the blocks outgrow 30 + 18 KiB: plain tables
+    "block-256": {"hip-block-size": 256},
+    "float64": {"hip-compute-type": "float64"},           # 32-byte entries: offsets do not fit eight bits, plain tables
+}
+
+
+@pytest.mark.parametrize("variant", sorted(GROUPED))
+def test_grouped_tables_on_the_discrete_configuration(native, variant):
+    """Tables read with the same index interleaved in blocks of four columns (one 16-byte read for up to four leaves):
+    the layout, the packed indices and every fallback to plain tables give the oracle's values."""
+    from spnc import synthetic as syn
+    c = syn.CONFIGS["c3"]
+    spn, X = c["spn"](), c["inputs"](4099)
+    X[5, :] = 77            # out of every feature's range
+    X[6, 3] = 9
+    k = compile_spn(native, spn, c["dtype"], marginal=False, **GROUPED[variant])
+    src = k.source()
+    grouped = variant not in ("plain", "no-room", "small-pool", "float64")
+    assert ("v_bfe_u32" in src) == grouped and ("spn_r4*" in src) == (grouped and variant != "singles"), variant
+    assert ("#define SPN_BLOCK 1024" in src) == (grouped and variant != "block-256")
+    got = run(k, X)
+    m = oracle_model(spn, c["dtype"])
+    if variant == "float64":
+        assert got.dtype == np.float64
+        ref = ev.ll_closed_f64(m, X, marginal=False)
+        assert np.array_equal(np.isneginf(got), np.isneginf(ref)) and np.isneginf(got[5]) and np.isneginf(got[6])
+        assert np.abs(got[np.isfinite(ref)] - ref[np.isfinite(ref)]).max() <= F64_TOL
+    else:
+        check_f32(got, m, X, False)
+        assert np.isneginf(got[5]) and np.isneginf(got[6])
+
+
+@pytest.mark.parametrize("dtype,marginal", [("uint8", False), ("int32", False), ("float32", True), ("float64", True)])
+def test_grouped_tables_feature_types_and_marginals(native, dtype, marginal):
+    """Small graph, grouping forced: every feature has five or six table leaves (one index each), joint tables for the
+    pairs inside the products; NaN selects the marginal entry, out-of-range values the impossible one."""
+    from spnc.structure import Categorical, Histogram, Product, Sum
+    rng = np.random.default_rng(23)
+    doms = [2, 3, 5, 4]
+    def product():
+        kids = [Categorical(p=list(rng.dirichlet(np.ones(d))), scope=f) for f, d in enumerate(doms)]
+        kids.append(Histogram(breaks=[0, 2, 3, 6], densities=list(rng.dirichlet(np.ones(3)) / np.array([2, 1, 3])), bin_repr_points=[1, 2, 4], scope=4))
+        return Product(children=kids)
+    spn = Sum(weights=list(rng.dirichlet(np.ones(2))), children=[
+        Sum(weights=list(rng.dirichlet(np.ones(3))), children=[product() for _ in range(3)]),
+        Sum(weights=list(rng.dirichlet(np.ones(2))), children=[product() for _ in range(2)])])
+    X = np.column_stack([rng.integers(0, d + 2, 700) for d in doms + [7]]).astype(dtype)
+    if marginal:
+        X[rng.random(X.shape) < 0.2] = np.nan
+        X[0, :] = np.nan
+    for opts in ({"hip-table-group-min-reads": 0}, {"hip-table-group-min-reads": 0, "hip-joint-tables": "false"}, {}):
+        k = compile_spn(native, spn, dtype, marginal=marginal, **opts)
+        assert ("spn_r4*" in k.source()) == bool(opts)
+        got = run(k, X)
+        check_f32(got, oracle_model(spn, dtype), X, marginal)
+        if marginal:
+            assert abs(got[0]) < 1e-6
+
+
 @pytest.mark.parametrize("kernel", ["jit", "interpreter"])
 def test_c5_marginal_in_f64(native, kernel):
     from spnc import synthetic as syn

@@ -229,6 +229,31 @@ def test_generated_source_variants(native):
     os.remove(k.fileName())
 
 
+def test_grouped_table_layout(native):
+    """Table-heavy graphs: tables read with the same index share blocks of four columns, indices are packed four to a
+    register, and the block size goes to 1024; small graphs and the option switch keep plain tables."""
+    from spnc import synthetic as syn
+    k = compile_spn(native, syn.c3_spn(), "int32", marginal=False)
+    src = k.source()
+    os.remove(k.fileName())
+    reads = src.count("*>(reinterpret_cast<const char*>(tab + ")
+    assert 600 < reads < 800 and src.count("const spn_r4 q") > 400 and src.count("v_bfe_u32") >= reads
+    assert "const unsigned P24 = " in src and "#define SPN_BLOCK 1024" in src and "__launch_bounds__(SPN_BLOCK, 1)" in src
+    pool = int(re.search(r"#define SPN_NTAB (\d+)", src).group(1))
+    assert pool % 4 == 0 and pool * 4 <= 80 * 1024
+    k = compile_spn(native, syn.c3_spn(), "int32", marginal=False, **{"hip-grouped-tables": "false"})
+    src = k.source()
+    os.remove(k.fileName())
+    assert "spn_r4 q" not in src and "v_bfe_u32" not in src and "#define SPN_BLOCK 256" in src and src.count("= tab[") == 1940
+    k = compile_spn(native, syn.c1_spn(), "int32", marginal=False)     # six tables, six indices: nothing to share
+    assert "v_bfe_u32" not in k.source()
+    os.remove(k.fileName())
+    with pytest.raises(RuntimeError, match="hip-table-group-window must not be negative"):
+        compile_spn(native, syn.c1_spn(), "int32", marginal=False, **{"hip-table-group-window": -1})
+    with pytest.raises(RuntimeError, match="hip-table-pad-kib must be in"):
+        compile_spn(native, syn.c1_spn(), "int32", marginal=False, **{"hip-table-pad-kib": 100})
+
+
 def test_kernel_file_round_trip(native):
     from spnc import synthetic as syn
     for opts in ({}, {"hip-kernel": "interpreter"}):
