@@ -26,12 +26,12 @@ FP64_VECTOR_PEAK_TFLOPS = 78.6   # MI355X FP64 vector, published
 # HBM bytes per launch from the counter runs summarised in profiles/<kernel>_<workload>.txt:
 # workload -> (samples per launch, bytes). Only valid for that launch size and the default options.
 MEASURED_HBM_TRAFFIC = {
-    "c1": (67108864, 1879038771),
-    "c2": (16777216, 1142146426),
-    "c3": (8388608, 3495354063),
-    "c4": (4194304, 5885434192),
-    "c5": (16777216, 1141489444),
-    "c5_f64": (16777216, 1210340704),
+    "c1": (67108864, 1879035700),
+    "c2": (16777216, 1142126559),
+    "c3": (8388608, 3394713247),
+    "c4": (4194304, 5892779431),
+    "c5": (16777216, 1141487599),
+    "c5_f64": (16777216, 1210338447),
 }
 
 
