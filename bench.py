@@ -121,7 +121,7 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None):
         "peak_note": ("published HBM3E bandwidth" if hbm_bound else
                       "published vector peak (FP32 157.3, FP64 78.6 TFLOP/s) counts an FMA as 2 flops; this path issues "
                       "single-flop instructions, so the ceiling is half of it in issue slots/s; achieved = (flops + "
-                      "3*transcendentals) per sample; a float64 exp/log is in fact ~22 instructions, not 4 slots"),
+                      "3*transcendentals) per sample; a float64 exp/log is in fact about 11 double-rate instructions and an LDS read, not 4 slots"),
         "fma_flops_tflops": round(tflops, 3),
         "kernel": "spn_kernel (hipRTC straight-line)" if info["kernel_kind"] == 1 else "spn_interp_kernel",
         "launch_ms": round(launch_ms, 4),
