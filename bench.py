@@ -26,12 +26,12 @@ FP64_VECTOR_PEAK_TFLOPS = 78.6   # MI355X FP64 vector, published
 # HBM bytes per launch from the counter runs summarised in profiles/<kernel>_<workload>.txt:
 # workload -> (samples per launch, bytes). Only valid for that launch size and the default options.
 MEASURED_HBM_TRAFFIC = {
-    "c1": (67108864, 1879035700),
-    "c2": (16777216, 1142126559),
-    "c3": (8388608, 3394713247),
-    "c4": (4194304, 5892779431),
-    "c5": (16777216, 1141487599),
-    "c5_f64": (16777216, 1210338447),
+    "c1": (67108864, 1879038771),
+    "c2": (16777216, 1142069219),
+    "c3": (8388608, 3394635282),
+    "c4": (4194304, 5884685364),
+    "c5": (16777216, 1141489239),
+    "c5_f64": (16777216, 1210340500),
 }
 
 
@@ -93,7 +93,9 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None):
 
     bytes_per_sample = cfg["features"] * info["bytes_per_feature"] + info["bytes_per_result"]
     flops, trans = info["flops_min"], info["trans_min"]
-    slots = flops + 3 * trans
+    # Issue slots: one per flop, four per transcendental, and one instead of two for every multiply-add pair that a
+    # fused instruction computes (Gaussian leaves and the product adds they feed), so that the fraction cannot pass 1.
+    slots = flops - info["fused_min"] + 3 * trans
     props = torch.cuda.get_device_properties(device)
     clock_hz = props.clock_rate * 1e3 if hasattr(props, "clock_rate") else 2.4e9
     # FP32 VALU issue rate: 128 lane-operations per CU per clock (a wave64 instruction issues in
@@ -120,14 +122,15 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None):
         "traffic": None,
         "peak_note": ("published HBM3E bandwidth" if hbm_bound else
                       "published vector peak (FP32 157.3, FP64 78.6 TFLOP/s) counts an FMA as 2 flops; this path issues "
-                      "single-flop instructions, so the ceiling is half of it in issue slots/s; achieved = (flops + "
-                      "3*transcendentals) per sample; a float64 exp/log is in fact about 11 double-rate instructions and an LDS read, not 4 slots"),
+                      "mostly single-flop instructions, so the ceiling is half of it in issue slots/s; achieved = (flops - fused "
+                      "multiply-add pairs + 3*transcendentals) per sample; a float64 exp/log is in fact about 11 double-rate instructions and an LDS read, not 4 slots"),
         "fma_flops_tflops": round(tflops, 3),
         "kernel": "spn_kernel (hipRTC straight-line)" if info["kernel_kind"] == 1 else "spn_interp_kernel",
         "launch_ms": round(launch_ms, 4),
         "bytes_per_sample": bytes_per_sample,
         "flops_per_sample": flops,
         "transcendentals_per_sample": trans,
+        "fused_multiply_adds_per_sample": info["fused_min"],
         "issue_slots_per_sample": slots,
         "valu_issue_peak_per_s": valu_peak,
         "valu_issue_frac": round(t_min_valu / t_launch, 4),

@@ -53,6 +53,8 @@ typedef struct spnc_hip_info {
   uint64_t trans_min;        /* of which transcendental */
   uint64_t flops_pairwise;   /* algorithmic flops per sample of the reference's pairwise trees */
   uint64_t trans_pairwise;
+  uint64_t fused_min;        /* multiply-add pairs among flops_min that one fused instruction computes in log space
+                                (Gaussian leaves and the product adds they feed): issue slots = flops_min - fused_min + 3 * trans_min */
 } spnc_hip_info;
 
 /* spn_compiler::isTargetSupported("HIP") (compiler/src/Driver.cpp:47-59): 1 if a gfx950 device

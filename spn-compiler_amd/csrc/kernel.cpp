@@ -325,6 +325,7 @@ void Kernel::fillInfo(spnc_hip_info* info) const {
   info->trans_min = stats_.transMin;
   info->flops_pairwise = stats_.flopsPairwise;
   info->trans_pairwise = stats_.transPairwise;
+  info->fused_min = stats_.fusedMin;
 }
 
 void Kernel::ensureDevice() {

@@ -310,6 +310,7 @@ Graph buildGraph(const RawQuery& q) {
         st.gaussians++;
         st.flopsMin += 4 + leafSelect;
         st.flopsPairwise += 4 + leafSelect;
+        st.fusedMin += 1;
         break;
       case NodeKind::Categorical:
         st.categoricals++;
@@ -326,6 +327,11 @@ Graph buildGraph(const RawQuery& q) {
         st.productAdds += k - 1;
         st.flopsMin += k - 1;
         st.flopsPairwise += k - 1;
+        {
+          uint64_t own = 0;  // Gaussian children read by this product only
+          for (uint32_t c : n.children) own += g.nodes[c].kind == NodeKind::Gaussian && g.nodes[c].uses == 1 ? 1 : 0;
+          st.fusedMin += std::min<uint64_t>(own, k ? k - 1 : 0);
+        }
         break;
       case NodeKind::Sum: {
         st.sums++;

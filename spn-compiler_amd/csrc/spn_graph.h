@@ -81,7 +81,11 @@ struct GraphStats {
   // Algorithmic work per sample: cheaper of pairwise tree (k==2) and n-ary LSE (k>=3) per sum,
   // 4 flops per Gaussian, 0 per table leaf, +1 select per leaf when marginal.
   uint64_t flopsMin = 0, transMin = 0, flopsPairwise = 0, transPairwise = 0;
-  uint64_t issueSlotsMin() const { return flopsMin + 3 * transMin; }
+  // Multiply-add pairs among flopsMin that one fused instruction computes in log space: a Gaussian leaf's
+  // (d*d)*den + coef, and the add of a product for every Gaussian child that only this product reads
+  // (den*(d*d + coef/den) + acc). Vector issue slots are priced without them, a transcendental at four slots.
+  uint64_t fusedMin = 0;
+  uint64_t issueSlotsMin() const { return flopsMin - fusedMin + 3 * transMin; }
 };
 
 struct Graph {

@@ -42,6 +42,7 @@ class _Info(ctypes.Structure):
         ("trans_min", ctypes.c_uint64),
         ("flops_pairwise", ctypes.c_uint64),
         ("trans_pairwise", ctypes.c_uint64),
+        ("fused_min", ctypes.c_uint64),
     ]
 
 

@@ -75,7 +75,7 @@ def test_algorithmic_counts(native):
     from spnc import synthetic as syn
     k = compile_spn(native, syn.c1_spn(), "int32")
     i = k.info()
-    assert (i["flops_min"], i["trans_min"], i["num_categorical"], i["product_adds"]) == (5, 0, 6, 5)
+    assert (i["flops_min"], i["trans_min"], i["num_categorical"], i["product_adds"], i["fused_min"]) == (5, 0, 6, 5, 0)
     os.remove(k.fileName())
     k = compile_spn(native, syn.c2_spn(), "float32")
     i = k.info()
@@ -83,6 +83,8 @@ def test_algorithmic_counts(native):
     assert (i["num_gaussian"], i["num_product"], i["num_sum"]) == (1024, 292, 73)
     assert (i["flops_min"], i["trans_min"]) == (4096 + 804 + 73 * 20, 73 * 5)
     assert (i["flops_pairwise"], i["trans_pairwise"]) == (4096 + 804 + 73 * 25, 73 * 6)
+    # fused multiply-adds: one inside every Gaussian leaf, and the 256 products of four leaves fold their three adds
+    assert i["fused_min"] == 1024 + 256 * 3 and i["fused_min"] < i["flops_min"]
     os.remove(k.fileName())
 
 
