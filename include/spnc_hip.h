@@ -55,6 +55,9 @@ typedef struct spnc_hip_info {
   uint64_t trans_pairwise;
   uint64_t fused_min;        /* multiply-add pairs among flops_min that one fused instruction computes in log space
                                 (Gaussian leaves and the product adds they feed): issue slots = flops_min - fused_min + 3 * trans_min */
+  unsigned feature_is_float; /* 1: inputs are IEEE floats of bytes_per_feature bytes; 0: unsigned integers of that width (signed
+                                integer arrays of the same width are read as unsigned, as the reference's index_cast / uitofp do) */
+  unsigned support_marginal; /* the query was compiled with NaN-marginalisation */
 } spnc_hip_info;
 
 /* spn_compiler::isTargetSupported("HIP") (compiler/src/Driver.cpp:47-59): 1 if a gfx950 device

@@ -385,8 +385,11 @@ struct Emitter {
                << x << " : " << L << "u;\n";
           if (g.supportMarginal) body << "  t" << f << " = (" << x << " != " << x << ") ? " << (L + 1) << "u : t" << f << ";\n";
         } else {
-          body << "  const unsigned t" << f << " = (" << x << " < (feat_t)" << L << ") ? (unsigned)" << x << " : " << L
-               << "u;\n";
+          // Compared in a type at least as wide as both sides: the table length cast to a narrow feature type
+          // would wrap (256 entries on an 8-bit feature).
+          const char* wide = g.ftype.bytes > 4 ? "(unsigned long long)" : "(unsigned)";
+          body << "  const unsigned t" << f << " = (" << wide << x << " < " << L << (g.ftype.bytes > 4 ? "ull" : "u") << ") ? (unsigned)" << x
+               << " : " << L << "u;\n";
         }
       }
     }

@@ -994,12 +994,6 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
     code_ptr ip = code;  // at the length word of the first instruction
     Head h = loadHead(codeGlobal, 0);
     R result;
-#ifdef SPN_INTERP_PROFILE
-    // Diagnostic build: cycles the first wave of the grid spends per instruction class on its third tile.
-    long long cyc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    int cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    long long t0 = clock64();
-#endif
     for (;;) {
       const uint32_t w0 = h.word(1);
       const bool spillPath = MODE == 2 || (MODE == 1 && (w0 & 0x80u));
@@ -1013,28 +1007,7 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
       else execute<R, LOG2, false, false>(ip + 1, h, Sl, a, tables, row, stagedMode, code, codeGlobal);
       ip = next;
       h = hn;
-#ifdef SPN_INTERP_PROFILE
-      {
-        const long long t1 = clock64();
-        const uint32_t op = w0 & 0x7fu;
-        int c = (op == OP_PROD || op == OP_PRODBATCH) ? 0 : (op == OP_OUTERSUM || op == OP_OUTERMM) ? ((((w0 >> 16) & 0xffu) == 8 ? 1 : 2) + (spillPath ? 2 : 0)) : 5;
-        if ((op == OP_PROD || op == OP_PRODBATCH) && spillPath) c = 6;
-        if (op == OP_LEAFMM || op == OP_LEAFPAIRMM) c = 7;
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
-          if (q == c) {
-            cyc[q] += t1 - t0;
-            cnt[q]++;
-          }
-        t0 = t1;
-      }
-#endif
     }
-#ifdef SPN_INTERP_PROFILE
-    if (blockIdx.x == 0 && threadIdx.x == 0 && base == 2 * lanes)
-      printf("profile: prod %d/%lld outer8 %d/%lld outer4 %d/%lld outer8-spill %d/%lld outer4-spill %d/%lld other %d/%lld prod-spill %d/%lld leaf %d/%lld\n",
-             cnt[0], cyc[0], cnt[1], cyc[1], cnt[2], cyc[2], cnt[3], cyc[3], cnt[4], cyc[4], cnt[5], cyc[5], cnt[6], cyc[6], cnt[7], cyc[7]);
-#endif
     if (valid) out[i] = Mt::finish(result);
   }
 }

@@ -101,6 +101,177 @@ InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
   return best;
 }
 
+// Walks a program as the kernel would and throws unless every access the kernel derives from it stays inside the
+// slot file, the table pool, the input row and the instruction itself. A program built here passes by
+// construction; one read back from a kernel file is only executed after it has passed.
+void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures) {
+  auto bad = [](const std::string& what, size_t at) -> void {
+    throw std::runtime_error("RUNTIME ERROR: malformed interpreter program (" + what + " at word " + std::to_string(at) + ")");
+  };
+  const std::vector<uint32_t>& c = p.code;
+  const size_t RW = p.f64 ? 2 : 1;
+  if (p.shortSlots > p.numSlots || p.numSlots > (1u << 20)) bad("slot counts", 0);
+  if (p.featureMode != FEAT_STAGED && p.featureMode != FEAT_DIRECT) bad("feature mode", 0);
+  if (p.f64 && p.log2Domain) bad("compute type", 0);
+  std::map<uint32_t, uint32_t> indexBound;  // staged index slot -> largest index it can hold
+  std::set<uint32_t> valueSlots;
+  for (const auto& sf : p.staged) {
+    if (sf.column >= numFeatures) bad("staged column", 0);
+    if (sf.valueSlot != NONE && sf.valueSlot >= p.numSlots) bad("staged value slot", 0);
+    if (sf.indexSlot != NONE && sf.indexSlot >= p.numSlots) bad("staged index slot", 0);
+    if (sf.tableLen > (1u << 24)) bad("staged table length", 0);
+    if (sf.valueSlot != NONE) valueSlots.insert(sf.valueSlot);
+    if (sf.indexSlot != NONE) indexBound[sf.indexSlot] = sf.tableLen + 1;
+  }
+  const bool staged = p.featureMode == FEAT_STAGED;
+  if (!staged && !p.staged.empty()) bad("staged features in a direct-feature program", 0);
+  size_t pc = 0;
+  for (;;) {
+    if (pc + 1 >= c.size()) bad("stream ends inside an instruction", pc);
+    const size_t len = c[pc], first = pc + 1, end = first + len;
+    if (len < 2 || end > c.size()) bad("length word", pc);
+    const uint32_t w0 = c[first], op = w0 & 0x7fu;
+    const bool flagged = (w0 & 0x80u) != 0;
+    auto need = [&](size_t words) {
+      if (words != len) bad("instruction length", pc);
+    };
+    auto slot = [&](size_t at) {
+      if (at >= end) bad("slot field outside its instruction", pc);
+      const uint32_t sl = c[at];
+      if (sl >= p.numSlots || (!flagged && sl >= p.shortSlots)) bad("slot number", at);
+      return sl;
+    };
+    // A list of n slots at `at`; tier 0 / 1 promise the short / long pool, `run` that the kernel may take the first
+    // number and count on from it.
+    auto list = [&](size_t at, size_t n, uint32_t tier, bool run) {
+      for (size_t j = 0; j < n; ++j) {
+        const uint32_t sl = slot(at + j);
+        if (run && sl != c[at] + j) bad("slot run", at + j);
+        if ((tier == 0 && sl >= p.shortSlots) || (tier == 1 && sl < p.shortSlots) || tier > 2) bad("slot tier", at + j);
+      }
+    };
+    auto feature = [&](size_t at, uint32_t tier) {
+      if (at >= end) bad("feature field outside its instruction", pc);
+      if (!staged) {
+        if (c[at] >= numFeatures) bad("feature column", at);
+        return;
+      }
+      const uint32_t sl = slot(at);
+      if (!valueSlots.count(sl)) bad("feature slot", at);
+      if ((tier == 0 && sl >= p.shortSlots) || (tier == 1 && sl < p.shortSlots) || tier > 2) bad("feature tier", at);
+    };
+    if (op == OP_END) {
+      need(2);
+      slot(first + 1);
+      if (end != c.size()) bad("words after the end instruction", end);
+      return;
+    }
+    if (len < 3) bad("instruction length", pc);
+    const uint32_t w1 = c[first + 1];
+    switch (op) {
+      case OP_PROD: {
+        if (first + 5 > end) bad("instruction length", pc);
+        const size_t ns = c[first + 2], ng = c[first + 3], nt = c[first + 4];
+        if (ns > len || ng > len || nt > len) bad("operand counts", pc);
+        need(5 + ns + ng * (1 + 3 * RW) + nt * 3);
+        slot(first + 1);
+        size_t q = first + 5;
+        for (size_t j = 0; j < ns; ++j) slot(q++);
+        for (size_t j = 0; j < ng; ++j, q += 1 + 3 * RW) feature(q, 2);
+        for (size_t j = 0; j < nt; ++j, q += 3) {
+          uint32_t bound;
+          if (staged) {
+            const auto it = indexBound.find(slot(q));
+            if (it == indexBound.end()) bad("table index slot", q);
+            bound = it->second;
+          } else {
+            if (c[q] >= numFeatures) bad("feature column", q);
+            bound = c[q + 2] + 1;
+          }
+          if (size_t(c[q + 1]) + bound >= p.tables.size()) bad("table offset", q + 1);
+        }
+        break;
+      }
+      case OP_PRODBATCH: {
+        const size_t n = w0 >> 8, G = w1 & 0xffu;
+        const uint32_t featTier = (w1 >> 8) & 3u, dstTier = (w1 >> 10) & 3u;
+        if (n < 2 || G < 1 || G > 4) bad("product batch shape", pc);
+        const size_t rec = 1 + G * (1 + 3 * RW);
+        need(2 + n * rec);
+        for (size_t i = 0; i < n; ++i) {
+          list(first + 2 + i * rec, 1, dstTier, false);
+          for (size_t j = 0; j < G; ++j) {
+            const size_t at = first + 2 + i * rec + 1 + j * (1 + 3 * RW);
+            feature(at, staged ? featTier : 2);
+            if (((w1 >> 12) & 1u) && i / 4 * 4 + 4 <= n && c[at] != c[first + 2 + (i / 4 * 4) * rec + 1 + j * (1 + 3 * RW)]) bad("grouped product batch", at);
+          }
+        }
+        break;
+      }
+      case OP_SUM: {
+        const size_t k = w0 >> 8;
+        if (k < 1) bad("sum without terms", pc);
+        need(2 + k * (1 + RW));
+        slot(first + 1);
+        for (size_t j = 0; j < k; ++j) slot(first + 2 + j * (1 + RW));
+        break;
+      }
+      case OP_SUMLAYER: {
+        const size_t k = w0 >> 8, m = w1;
+        if (k < 1 || !(m == 2 || m == 4 || m == 8)) bad("sum layer shape", pc);
+        need(2 + m + k + k * m * RW);
+        for (size_t j = 0; j < m + k; ++j) slot(first + 2 + j);
+        break;
+      }
+      case OP_OUTERSUM: {
+        const size_t na = (w0 >> 8) & 0xffu, nb = (w0 >> 16) & 0xffu, m = w1;
+        if (na < 1 || !(nb == 2 || nb == 4 || nb == 8 || nb == 16) || !(m == 2 || m == 4 || m == 8) || (w0 >> 24)) bad("outer sum shape", pc);
+        need(2 + m + na + nb + na * nb * m * RW);
+        for (size_t j = 0; j < m + na + nb; ++j) slot(first + 2 + j);
+        break;
+      }
+      case OP_OUTERMM: {
+        const uint32_t na = (w0 >> 8) & 0xffu, nb = (w0 >> 16) & 0xffu;
+        if (p.f64 || !matrixFormShape(na, nb) || (w1 & 0xffu) != 8 || (w1 >> 12)) bad("matrix-form outer sum shape", pc);
+        need(2 + 8 + na + nb + 3 + size_t(na) * nb * 8);
+        const size_t dst = first + 2, as = dst + 8, bs = as + na, scales = bs + nb;
+        list(dst, 8, (w0 >> 28) & 3u, (w1 >> 11) & 1u);
+        list(as, na, (w0 >> 24) & 3u, (w1 >> 9) & 1u);
+        list(bs, nb, (w0 >> 26) & 3u, (w1 >> 10) & 1u);
+        if ((w1 >> 8) & 1u) slot(scales);
+        if ((w0 >> 30) & 1u) slot(scales + 1);
+        if ((w0 >> 31) & 1u) slot(scales + 2);
+        break;
+      }
+      case OP_LEAFMM:
+      case OP_LEAFPAIRMM:
+      case OP_LEAFQUADMM: {
+        const uint32_t na = (w0 >> 8) & 0xffu, nb = (w0 >> 16) & 0xffu, G = (w1 >> 12) & 0xfu, featTier = (w1 >> 16) & 3u;
+        if (p.f64 || (w1 & 0xffu) != 8) bad("leaf region shape", pc);
+        size_t regions, products, weights;
+        if (op == OP_LEAFMM) {
+          if (!((na == 4 && nb == 4) || (na == 8 && nb == 8)) || !(G == 1 || G == 2 || G == 4)) bad("leaf region shape", pc);
+          regions = 1, products = na + nb, weights = size_t(na) * nb * 8;
+        } else if (op == OP_LEAFPAIRMM) {
+          if (na != 4 || nb != 0 || !(G == 1 || G == 2 || G == 4)) bad("leaf region pair shape", pc);
+          regions = 2, products = 16, weights = 2 * 128 + 512;
+        } else {
+          if (na != 4 || nb != 0 || !(G == 1 || G == 2)) bad("leaf region quad shape", pc);
+          regions = 4, products = 32, weights = 2 * (2 * 128 + 512) + 512;
+        }
+        need(2 + 8 + 1 + 2 * regions * G + products * G * 3 + weights);
+        list(first + 2, 8, (w0 >> 28) & 3u, (w1 >> 11) & 1u);
+        if ((w1 >> 8) & 1u) slot(first + 10);
+        for (size_t j = 0; j < 2 * regions * G; ++j) feature(first + 11 + j, staged ? featTier : 2);
+        break;
+      }
+      default:
+        bad("opcode", first);
+    }
+    pc = end;
+  }
+}
+
 namespace {
 InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t longRange, bool stagedLong) {
   if (!o.useLogSpace) throw std::runtime_error("The interpreter kernel supports log-space computation only");

@@ -86,4 +86,8 @@ struct InterpProgram {
 
 InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o);
 
+// Throws std::runtime_error unless every slot, table, feature and weight access the kernel derives from the program
+// stays in range (slot numbers and their tier flags, table offsets, feature columns, instruction lengths).
+void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures);
+
 }  // namespace spnc_hip

@@ -112,6 +112,18 @@ struct Reader {
   }
 };
 
+// Shortest decimal form that reads back as the same double, integral values with ".0" (2.0, 4.4).
+std::string jsonDouble(double v) {
+  char buf[40];
+  for (int prec = 1; prec <= 17; ++prec) {
+    std::snprintf(buf, sizeof(buf), "%.*g", prec, v);
+    if (std::strtod(buf, nullptr) == v) break;
+  }
+  std::string t(buf);
+  if (t.find_first_of(".eEn") == std::string::npos) t += ".0";
+  return t;
+}
+
 std::string makeKernelFilePath() {
   const char* dir = std::getenv("TMPDIR");
   std::string tmpl = std::string(dir && *dir ? dir : "/tmp") + "/spnc_hip_XXXXXX.hipk";
@@ -157,6 +169,7 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
   if (useInterp) {
     k->kind_ = SPNC_HIP_KERNEL_INTERPRETER;
     k->prog_ = buildInterpProgram(g, o);
+    checkInterpProgram(k->prog_, g.numFeatures);  // the builder's invariants, checked before anything runs on a device
     k->bytesPerResult_ = k->prog_.f64 ? 8 : 4;
     k->inputAlign_ = g.ftype.bytes;
     k->text_ = k->prog_.listing;
@@ -180,13 +193,21 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
   }
   if (o.dumpIR) std::cerr << "// *** device code for " << k->kernelName_ << " ***\n" << k->text_ << std::endl;
   if (o.collectGraphStats) {
-    std::ofstream st(o.graphStatsFile);
+    // The reference's keys and its compact, key-sorted JSON (LoSPNGraphStatsCollection.cpp:85-102), counted as there
+    // on the binarised graph before identical nodes are merged; "hip" holds what this target adds.
+    const LoSpnStats ls = computeLoSpnStats(q, o.useLogSpace);
     const GraphStats& s = g.stats;
-    st << "{\"featureCount\": " << g.numFeatures << ", \"sumCount\": " << s.sums << ", \"productCount\": " << s.products
-       << ", \"histogramCount\": " << s.histograms << ", \"categoricalCount\": " << s.categoricals << ", \"gaussianCount\": " << s.gaussians
-       << ", \"innerCount\": " << (s.sums + s.products) << ", \"leafCount\": " << (s.histograms + s.categoricals + s.gaussians)
-       << ", \"maxFanIn\": " << s.maxFanIn << ", \"sumTerms\": " << s.sumTerms << ", \"flopsMin\": " << s.flopsMin
-       << ", \"transMin\": " << s.transMin << "}\n";
+    std::ofstream st(o.graphStatsFile);
+    if (!st) fatal("COMPILATION ERROR: cannot write graph statistics to '" + o.graphStatsFile + "'");
+    st << "{\"averageDepth\":" << jsonDouble(ls.averageDepth) << ",\"categoricalCount\":" << ls.categoricalCount
+       << ",\"constantCount\":" << ls.constantCount << ",\"featureCount\":" << g.numFeatures << ",\"gaussianCount\":" << ls.gaussianCount
+       << ",\"hip\":{\"depthsExact\":" << (ls.depthsExact ? "true" : "false") << ",\"flopsMin\":" << s.flopsMin << ",\"maxFanIn\":" << s.maxFanIn
+       << ",\"mergedNodes\":" << g.nodes.size() << ",\"sumTerms\":" << s.sumTerms << ",\"transMin\":" << s.transMin << "}"
+       << ",\"histogramCount\":" << ls.histogramCount << ",\"innerCount\":" << ls.innerCount() << ",\"leafCount\":" << ls.leafCount()
+       << ",\"maxDepth\":" << ls.maxDepth << ",\"medianDepth\":" << jsonDouble(ls.medianDepth) << ",\"minDepth\":" << ls.minDepth
+       << ",\"productCount\":" << ls.productCount << ",\"sumCount\":" << ls.sumCount << "}";
+    st.close();
+    if (!st) fatal("COMPILATION ERROR: cannot write graph statistics to '" + o.graphStatsFile + "'");
   }
   k->fileName_ = makeKernelFilePath();
   k->save(k->fileName_);
@@ -293,6 +314,24 @@ std::unique_ptr<Kernel> Kernel::load(const std::string& kernelFile) {
   } else {
     fatal("RUNTIME ERROR: unknown kernel kind in " + kernelFile);
   }
+  // Nothing read from the file reaches a launch unchecked: a truncated, foreign or damaged file is a host error.
+  auto reject = [&](const char* what) { fatal("RUNTIME ERROR: kernel file " + kernelFile + " is damaged (" + what + ")"); };
+  if (r.pos != buf.size()) reject("trailing bytes");
+  if (k->numFeatures_ == 0 || k->numFeatures_ > (1u << 24)) reject("feature count");
+  if (k->featureType_ > unsigned(FeatureType::F64)) reject("feature type");
+  static const unsigned widths[] = {1, 2, 4, 8, 4, 8};
+  if (k->bytesPerFeature_ != widths[k->featureType_]) reject("feature width");
+  if (k->bytesPerResult_ != 4 && k->bytesPerResult_ != 8) reject("result width");
+  if (k->kind_ == SPNC_HIP_KERNEL_JIT) {
+    if (k->blockSize_ < 64 || k->blockSize_ > 1024 || k->blockSize_ % 64 != 0) reject("block size");
+    if (k->samplesPerLane_ < 1 || k->samplesPerLane_ > 16) reject("samples per lane");
+    if (k->inputAlign_ == 0 || k->inputAlign_ > 16 || (k->inputAlign_ & (k->inputAlign_ - 1)) != 0) reject("input alignment");
+    if (k->gridPolicy_ < -1 || k->gridPolicy_ > 64) reject("grid policy");
+    if (k->entry_.empty() || k->codeObject_.size() < 64) reject("code object");
+  } else {
+    if (k->bytesPerResult_ != (k->prog_.f64 ? 8u : 4u)) reject("result width");
+    checkInterpProgram(k->prog_, k->numFeatures_);
+  }
   return k;
 }
 
@@ -326,10 +365,22 @@ void Kernel::fillInfo(spnc_hip_info* info) const {
   info->flops_pairwise = stats_.flopsPairwise;
   info->trans_pairwise = stats_.transPairwise;
   info->fused_min = stats_.fusedMin;
+  info->feature_is_float = featureType_ == unsigned(FeatureType::F32) || featureType_ == unsigned(FeatureType::F64);
+  info->support_marginal = marginal_ ? 1u : 0u;
 }
 
 void Kernel::ensureDevice() {
   if (deviceReady_) return;
+  try {
+    prepareDevice();
+  } catch (...) {
+    releaseDevice();  // nothing half-built stays behind: the next call starts from scratch
+    throw;
+  }
+  deviceReady_ = true;
+}
+
+void Kernel::prepareDevice() {
   int count = 0;
   if (hipGetDeviceCount(&count) != hipSuccess || count == 0) fatal("RUNTIME ERROR: no HIP device available");
   hipCheck(hipGetDevice(&device_), "hipGetDevice");
@@ -397,7 +448,6 @@ void Kernel::ensureDevice() {
     spillBytes_ = size_t(prog_.numSlots - ldsSlots_) * lanes * rb;
     if (spillBytes_) hipCheck(hipMalloc(&dSpill_, spillBytes_), "hipMalloc(spill)");
   }
-  deviceReady_ = true;
 }
 
 void Kernel::releaseDevice() {
@@ -472,13 +522,18 @@ void Kernel::executeDevice(size_t n, const void* dIn, void* dOut, hipStream_t st
 
 void Kernel::ensureStaging(size_t rows) {
   if (rows <= stageRows_) return;
+  // The old buffers go first and the row count with them, so that a failed allocation below leaves
+  // "no staging buffers" behind, never a count that promises more than the pointers hold.
+  stageRows_ = 0;
   for (auto& s : stage_) {
     if (s.hIn) (void)hipHostFree(s.hIn);
     if (s.hOut) (void)hipHostFree(s.hOut);
     if (s.dIn) (void)hipFree(s.dIn);
     if (s.dOut) (void)hipFree(s.dOut);
     s.hIn = s.hOut = s.dIn = s.dOut = nullptr;
-    const size_t inBytes = rows * numFeatures_ * bytesPerFeature_, outBytes = rows * bytesPerResult_;
+  }
+  const size_t inBytes = rows * numFeatures_ * bytesPerFeature_, outBytes = rows * bytesPerResult_;
+  for (auto& s : stage_) {
     hipCheck(hipHostMalloc(&s.hIn, inBytes, hipHostMallocDefault), "hipHostMalloc(input staging)");
     hipCheck(hipHostMalloc(&s.hOut, outBytes, hipHostMallocDefault), "hipHostMalloc(output staging)");
     hipCheck(hipMalloc(&s.dIn, inBytes), "hipMalloc(input)");

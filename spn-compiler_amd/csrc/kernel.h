@@ -42,6 +42,7 @@ class Kernel {
   Kernel() = default;
   void save(const std::string& path) const;
   void ensureDevice();
+  void prepareDevice();
   void releaseDevice();
   void ensureStaging(size_t rows);
   void launch(size_t n, const void* dIn, void* dOut, hipStream_t stream);

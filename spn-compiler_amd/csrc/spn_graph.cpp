@@ -442,4 +442,161 @@ Graph buildGraph(const RawQuery& q) {
   return g;
 }
 
+namespace {
+
+// Depth of operand i below the top operation of a balanced binary tree over k operands with pivot ceil(k/2)
+// (mlir/lib/Conversion/HiSPNtoLoSPN/NodePatterns.cpp:17-40,49-88); a tree over one operand is that operand.
+int treeDepth(size_t k, size_t i) {
+  int d = 0;
+  while (k > 2) {
+    const size_t pivot = (k + 1) / 2;
+    if (i < pivot) {
+      k = pivot;
+    } else {
+      i -= pivot;
+      k -= pivot;
+    }
+    ++d;
+  }
+  return k == 2 ? d + 1 : d;
+}
+
+}  // namespace
+
+LoSpnStats computeLoSpnStats(const RawQuery& q, bool logSpace) {
+  const RawModel& m = q.model;
+  LoSpnStats st;
+  std::unordered_map<int32_t, size_t> byId;
+  for (size_t i = 0; i < m.nodes.size(); ++i) {
+    const RawNode& n = m.nodes[i];
+    byId[n.id] = i;
+    const uint64_t k = n.children.size();
+    switch (n.kind) {
+      case NodeKind::Product: st.productCount += k ? k - 1 : 0; break;
+      case NodeKind::Sum:
+        st.sumCount += k ? k - 1 : 0;
+        st.productCount += k;
+        st.constantCount += k;
+        break;
+      case NodeKind::Categorical: st.categoricalCount++; break;
+      case NodeKind::Gaussian: st.gaussianCount++; break;
+      case NodeKind::Histogram: st.histogramCount++; break;
+    }
+  }
+  // Leaf depths as the reference's SPNNodeLevel takes them (mlir/lib/Dialect/LoSPN/Analysis/SPNNodeLevel.cpp:19-97): a walk
+  // from the root along every path, operands in order; an operation met again takes the larger of its old and new
+  // level and hands that on, and a leaf is counted once per path that reaches it. Only the top operation of a
+  // node's binary tree needs a stored level: the operations inside the tree follow it at fixed offsets.
+  auto childDepth = [&](const RawNode& n, size_t i) { return treeDepth(n.children.size(), i) + (n.kind == NodeKind::Sum ? 1 : 0); };
+  auto isLeaf = [](const RawNode& n) { return n.kind != NodeKind::Product && n.kind != NodeKind::Sum; };
+  const int rootLevel = logSpace ? 0 : 1;
+  std::map<int, double> histogram;  // leaf level -> visits
+  double visits = 0;
+  const auto rootIt = byId.find(m.rootNode);
+  if (rootIt == byId.end()) return st;
+  {
+    std::vector<int> level(m.nodes.size(), -1);
+    struct Frame {
+      size_t node;
+      int level;
+      size_t next;
+    };
+    std::vector<Frame> stack;
+    const double budget = 2e7;
+    auto enter = [&](size_t node, int incoming) {
+      const RawNode& n = m.nodes[node];
+      // A product over one operand is that operand: it has no operation of its own.
+      int lv = incoming;
+      if (level[node] >= 0 && level[node] != incoming) lv = std::max(incoming, level[node]);
+      level[node] = lv;
+      if (isLeaf(n)) {
+        histogram[lv] += 1;
+        visits += 1;
+      } else {
+        stack.push_back({node, lv, 0});
+      }
+    };
+    enter(rootIt->second, rootLevel);
+    double steps = 0;
+    while (!stack.empty() && steps <= budget) {
+      Frame& f = stack.back();
+      const RawNode& n = m.nodes[f.node];
+      if (f.next >= n.children.size()) {
+        stack.pop_back();
+        continue;
+      }
+      const size_t i = f.next++;
+      const auto it = byId.find(n.children[i]);
+      if (it == byId.end()) continue;
+      ++steps;
+      enter(it->second, f.level + childDepth(n, i));
+    }
+    if (!stack.empty()) {
+      // Heavily shared graphs (region graphs) have more root-to-leaf paths than anyone can walk. Their leaves are
+      // then counted per path by recurrence over the graph, each at its path length, without the
+      // larger-level-on-revisit rule of the walk, whose outcome depends on the order of the visits.
+      st.depthsExact = false;
+      histogram.clear();
+      std::vector<std::map<int, double>> below(m.nodes.size());  // node -> (leaf depth below the node's top operation -> paths)
+      std::vector<char> done(m.nodes.size(), 0);
+      std::vector<std::pair<size_t, size_t>> work{{rootIt->second, 0}};
+      while (!work.empty()) {
+        auto& [node, next] = work.back();
+        const RawNode& n = m.nodes[node];
+        if (done[node]) {
+          work.pop_back();
+          continue;
+        }
+        if (isLeaf(n)) {
+          below[node][0] = 1;
+          done[node] = 1;
+          work.pop_back();
+          continue;
+        }
+        if (next < n.children.size()) {
+          const auto it = byId.find(n.children[next++]);
+          if (it != byId.end() && !done[it->second]) work.push_back({it->second, 0});
+          continue;
+        }
+        for (size_t i = 0; i < n.children.size(); ++i) {
+          const auto it = byId.find(n.children[i]);
+          if (it == byId.end()) continue;
+          for (const auto& [d, cnt] : below[it->second]) below[node][d + childDepth(n, i)] += cnt;
+        }
+        done[node] = 1;
+        work.pop_back();
+      }
+      for (const auto& [d, cnt] : below[rootIt->second]) histogram[d + rootLevel] = cnt;
+    }
+  }
+  if (histogram.empty()) return st;
+  st.minDepth = histogram.begin()->first;
+  st.maxDepth = histogram.rbegin()->first;
+  double total = 0, weighted = 0;
+  for (const auto& [d, cnt] : histogram) {
+    total += cnt;
+    weighted += d * cnt;
+  }
+  st.averageDepth = weighted / total;
+  // The median as the reference finds it (SPNNodeLevel.cpp:43-60): the level whose bucket holds position n/2, and for an
+  // even count whose position n/2+1 closes that bucket, the mean of that level and the next one. Where no next level
+  // exists the reference reads past its set of levels; with its standard library that read yields the number of
+  // distinct levels, which is what its own test expects (two leaves at depth 2: median 1.5) and what is kept here.
+  const double pivot = total / 2.0;
+  double index = 0;
+  for (auto it = histogram.begin(); it != histogram.end(); ++it) {
+    index += it->second;
+    if (pivot < index && pivot > index - it->second) {
+      if (std::fmod(total, 2.0) == 0 && double((long long)(pivot + 1)) == index) {
+        auto nextBucket = std::next(it);
+        const double nextLevel = nextBucket != histogram.end() ? double(nextBucket->first) : double(histogram.size());
+        st.medianDepth = (double(it->first) + nextLevel) / 2.0;
+      } else {
+        st.medianDepth = it->first;
+      }
+    }
+  }
+  return st;
+}
+
 }  // namespace spnc_hip

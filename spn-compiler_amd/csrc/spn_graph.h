@@ -88,6 +88,24 @@ struct GraphStats {
   uint64_t issueSlotsMin() const { return flopsMin - fusedMin + 3 * transMin; }
 };
 
+// What the reference's "collect-graph-stats" pass reports (mlir/lib/Dialect/LoSPN/Passes/LoSPNGraphStatsCollection.cpp:44-97):
+// operation counts of the binarised LoSPN graph right after the HiSPN lowering, i.e. before any merging of
+// identical nodes, and the depths of its leaves.
+struct LoSpnStats {
+  uint64_t sumCount = 0;       // binary adds: k-1 per k-ary sum
+  uint64_t productCount = 0;   // binary multiplies: k-1 per k-ary product and one per weighted sum term
+  uint64_t constantCount = 0;  // weight constants: one per sum term
+  uint64_t categoricalCount = 0, gaussianCount = 0, histogramCount = 0;
+  uint64_t innerCount() const { return sumCount + productCount; }
+  uint64_t leafCount() const { return categoricalCount + gaussianCount + histogramCount + constantCount; }  // constants count as leaves there
+  int minDepth = 0, maxDepth = 0;
+  double averageDepth = 0, medianDepth = 0;
+  bool depthsExact = true;     // false: the graph shares so many nodes that the reference's path-by-path walk was replaced (see computeLoSpnStats)
+};
+
+// logSpace false adds the final log operation as the root of the depth count, as the reference's linear-space lowering does.
+LoSpnStats computeLoSpnStats(const RawQuery& q, bool logSpace);
+
 struct Graph {
   std::string name;
   FeatureTypeInfo ftype;

@@ -43,6 +43,8 @@ class _Info(ctypes.Structure):
         ("flops_pairwise", ctypes.c_uint64),
         ("trans_pairwise", ctypes.c_uint64),
         ("fused_min", ctypes.c_uint64),
+        ("feature_is_float", ctypes.c_uint),
+        ("support_marginal", ctypes.c_uint),
     ]
 
 
@@ -149,8 +151,10 @@ class Kernel:
 
     def execute(self, num_elements, inputs):
         """[num_elements, numFeatures] host array in -> [num_elements] log-likelihoods out."""
-        if inputs.dtype.itemsize != self.bytesPerFeature():
-            raise RuntimeError(f"Input dtype {inputs.dtype} does not match the kernel's {self.bytesPerFeature()}-byte feature type")
+        want = ("float" if self._info.feature_is_float else "int") + str(8 * self.bytesPerFeature())
+        if inputs.dtype.itemsize != self.bytesPerFeature() or (inputs.dtype.kind == "f") != bool(self._info.feature_is_float) \
+                or inputs.dtype.kind not in "fiu":
+            raise RuntimeError(f"Input dtype {inputs.dtype} does not match the kernel's feature type {want}")
         if inputs.ndim != 2 or inputs.shape[1] != self.numFeatures() or inputs.shape[0] < num_elements:
             raise RuntimeError(f"Input must have shape [{num_elements}, {self.numFeatures()}], got {inputs.shape}")
         inputs = np.ascontiguousarray(inputs)
@@ -187,7 +191,22 @@ class SPNCompiler:
 
     @staticmethod
     def isFeatureAvailable(feature):
-        return False
+        """Host CPU features by the reference's names (compiler/src/Driver.cpp:61-82): "vectorize", "AVX", "AVX2",
+        "AVX512", "Neon"; anything else is False. Read from the kernel's CPU flags; the HIP kernels do not depend on
+        them, the query exists so that callers written against the reference keep working."""
+        flags = set()
+        try:
+            with open("/proc/cpuinfo") as f:
+                for line in f:
+                    if line.lower().startswith(("flags", "features")):
+                        flags.update(line.split(":", 1)[1].split())
+                        break
+        except OSError:
+            return False
+        have = {"AVX": "avx" in flags, "AVX2": "avx2" in flags, "AVX512": "avx512f" in flags,
+                "Neon": bool(flags & {"neon", "asimd"})}
+        have["vectorize"] = any(have.values())
+        return bool(have.get(feature, False))
 
     @staticmethod
     def getHostArchitecture():

@@ -70,9 +70,15 @@ def c3_domains(num_features=100, seed=3):
     return doms
 
 
-def c3_spn(num_features=100, seed=3):
+def c3_spn(num_features=100, seed=3, sum_levels=2, inner_fan_in=(2, 9)):
+    """Discrete SPN over `num_features` features: sums and products alternate from a sum root; every sum draws
+    2 to 8 children with Dirichlet(1) weights; a product splits its scope into 2 or 3 random parts, one sum (or a
+    single leaf) per part, until `sum_levels` levels of sums exist or the scope is small, where the product factorises
+    into the leaves of its scope. Defaults: 1651 nodes (10 sums, 40 products, 1601 leaves).
+    ``c3_deep_spn`` is the deeper, narrower variant (68 sums of 2 to 4 children, 2640 nodes)."""
     doms = c3_domains(num_features, seed)
     rng = np.random.default_rng(seed + 1000)
+    max_level = 2 * sum_levels - 1
 
     def leaf(f):
         kind, d = doms[f]
@@ -83,7 +89,7 @@ def c3_spn(num_features=100, seed=3):
         return Categorical(p=[float(v) for v in p], scope=int(f))
 
     def make_product(scope, level):
-        if len(scope) <= 6 or level >= 5:
+        if len(scope) <= 6 or level >= max_level:
             return Product(children=[leaf(f) for f in scope])
         parts = int(rng.integers(2, 4))
         perm = [scope[i] for i in rng.permutation(len(scope))]
@@ -95,11 +101,16 @@ def c3_spn(num_features=100, seed=3):
         return Product(children=children)
 
     def make_sum(scope, level):
-        k = int(rng.integers(2, 9)) if level == 0 else int(rng.integers(2, 4))
+        k = int(rng.integers(2, 9)) if level == 0 else int(rng.integers(*inner_fan_in))
         weights = rng.dirichlet(np.ones(k))
         return Sum(weights=[float(w) for w in weights], children=[make_product(scope, level + 1) for _ in range(k)])
 
     return make_sum(list(range(num_features)), 0)
+
+
+def c3_deep_spn(num_features=100, seed=3):
+    """Three levels of sums, inner sums of 2 or 3 children: 68 sums, 174 products, 2398 leaves."""
+    return c3_spn(num_features, seed, sum_levels=3, inner_fan_in=(2, 4))
 
 
 def c3_inputs(n, num_features=100, seed=3, data_seed=103):
@@ -153,6 +164,8 @@ CONFIGS = {
                desc="random depth-6 sum/product tree, 16 Gaussian features, float32 [N,16]"),
     "c3": dict(spn=c3_spn, inputs=c3_inputs, dtype="int32", marginal=False, n=8 * 2 ** 20, features=100,
                desc="discrete SPN, 100 features, Categorical + Histogram leaves, int32 [N,100]"),
+    "c3_deep": dict(spn=c3_deep_spn, inputs=c3_inputs, dtype="int32", marginal=False, n=8 * 2 ** 20, features=100,
+                    desc="discrete SPN, 100 features, three levels of narrow sums (2640 nodes), int32 [N,100]"),
     "c4": dict(spn=c4_spn, inputs=c4_inputs, dtype="float32", marginal=False, n=4 * 2 ** 20, features=32,
                desc="RAT-SPN-style region graph, 32 Gaussian features, 10 repetitions, float32 [N,32]"),
     "c5": dict(spn=c2_spn, inputs=c5_inputs, dtype="float32", marginal=True, n=16 * 2 ** 20, features=16,

@@ -98,7 +98,7 @@ def test_hipcompiler_argument_checks(native):
         c.execute(k, "nope")
     with pytest.raises(RuntimeError, match="Input must be a two-dimensional array"):
         c.execute(k, np.zeros((2, 3, 6), dtype=np.int32))
-    with pytest.raises(RuntimeError, match="does not match the kernel's 4-byte feature type"):
+    with pytest.raises(RuntimeError, match="does not match the kernel's feature type int32"):
         c.execute(k, np.zeros((4, 6), dtype=np.float64))
     with pytest.raises(RuntimeError, match=r"Input must have shape \[4, 6\]"):
         c.execute(k, np.zeros((4, 5), dtype=np.int32))

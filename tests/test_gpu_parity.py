@@ -132,7 +132,7 @@ def test_golden_outputs_f64(native, tmp_path, name, opts):
 
 
 @pytest.mark.parametrize("variant", sorted(VARIANTS))
-@pytest.mark.parametrize("cfg", ["c1", "c2", "c3", "c4", "c5"])
+@pytest.mark.parametrize("cfg", ["c1", "c2", "c3", "c3_deep", "c4", "c5"])
 def test_benchmark_configurations(native, cfg, variant):
     from spnc import synthetic as syn
     c = syn.CONFIGS[cfg]
@@ -159,12 +159,13 @@ GROUPED = {
 }
 
 
+@pytest.mark.parametrize("cfg", ["c3", "c3_deep"])
 @pytest.mark.parametrize("variant", sorted(GROUPED))
-def test_grouped_tables_on_the_discrete_configuration(native, variant):
+def test_grouped_tables_on_the_discrete_configuration(native, variant, cfg):
     """Tables read with the same index interleaved in blocks of four columns (one 16-byte read for up to four leaves):
     the layout, the packed indices and every fallback to plain tables give the oracle's values."""
     from spnc import synthetic as syn
-    c = syn.CONFIGS["c3"]
+    c = syn.CONFIGS[cfg]
     spn, X = c["spn"](), c["inputs"](4099)
     X[5, :] = 77            # out of every feature's range
     X[6, 3] = 9

@@ -115,12 +115,150 @@ def test_option_handling(native):
 
 
 def test_graph_stats_file(native, tmp_path):
+    """collect-graph-stats writes the reference's keys, counted on the binarised graph
+    (mlir/lib/Dialect/LoSPN/Passes/LoSPNGraphStatsCollection.cpp:85-97)."""
     import json
+    from spnc.structure import Histogram, Product
+    keys = {"featureCount", "minDepth", "maxDepth", "averageDepth", "medianDepth", "innerCount", "leafCount", "sumCount", "productCount",
+            "categoricalCount", "constantCount", "gaussianCount", "histogramCount"}
     out = tmp_path / "stats.json"
-    k = compile_query(native, os.path.join(GOLDEN, "NIPS5.bin"), **{"collect-graph-stats": "true", "graph-stats-file": str(out)})
-    st = json.load(open(out))
-    assert (st["featureCount"], st["sumCount"], st["productCount"], st["histogramCount"], st["innerCount"], st["leafCount"]) == (5, 1, 2, 10, 3, 10)
+    stats_opts = {"collect-graph-stats": "true", "graph-stats-file": str(out)}
+
+    def stats(kernel):
+        os.remove(kernel.fileName())
+        text = open(out).read()
+        st = json.loads(text)
+        assert keys <= set(st) and set(st) - keys == {"hip"}
+        assert list(st) == sorted(st) and " " not in text      # the reference's JSON writer sorts keys and prints compactly
+        return st
+
+    # NIPS5 by hand: one sum over two products of five histograms = 13 nodes. Binarised: 1 add, 2 weight multiplies with 2
+    # constants, 2 * 4 product multiplies; leaf depths below a product of five are 3,3,2,2,2 and the product's top
+    # multiply sits at level 2 (add, weight multiply, product).
+    st = stats(compile_query(native, os.path.join(GOLDEN, "NIPS5.bin"), **stats_opts))
+    assert (st["featureCount"], st["sumCount"], st["productCount"], st["constantCount"], st["histogramCount"]) == (5, 1, 10, 2, 10)
+    assert (st["innerCount"], st["leafCount"], st["gaussianCount"], st["categoricalCount"]) == (11, 12, 0, 0)
+    assert (st["minDepth"], st["maxDepth"], st["averageDepth"], st["medianDepth"]) == (4, 5, 4.4, 4.5)
+    assert st["hip"]["depthsExact"] is True and st["hip"]["mergedNodes"] == 13
+
+    # The reference's own expectations: mlir/test/analysis/lospn/lospn-graph-stats-collection-sum.mlir:50-63 (a sum over five
+    # categoricals, linear space, so the final log is the root) and ...-mul.mlir:34-48 (a product of two histograms).
+    # (that sum mixes scopes, which the serializer of this package refuses, so its file is written field by field)
+    probs = [[.35, .55, .1], [.25, .625, .125], [.5, .2, .3], [.6, .15, .25], [.8, .14, .06]]
+    path = rf.write(str(tmp_path / "sum.bin"), nodes=[rf.cat(i + 1, i, p=p) for i, p in enumerate(probs)] +
+                    [rf.wsum(0, [1, 2, 3, 4, 5], [.1, .1, .1, .4, .3])], scope=[0, 1, 2, 3, 4], feature_type="int32")
+    st = stats(compile_query(native, path, **stats_opts, **{"use-log-space": "false"}))
+    want = {"averageDepth": 4.4, "categoricalCount": 5, "constantCount": 5, "featureCount": 5, "gaussianCount": 0, "histogramCount": 0,
+            "innerCount": 9, "leafCount": 10, "maxDepth": 5, "medianDepth": 4, "minDepth": 4, "productCount": 5, "sumCount": 4}
+    assert {k_: st[k_] for k_ in want} == want
+    hists = [Histogram([0., 1., 2.], [0.25, 0.75], [1, 1], scope=0), Histogram([0., 1., 2.], [0.45, 0.55], [1, 1], scope=1)]
+    st = stats(compile_spn(native, Product(children=hists), "int32", **stats_opts, **{"use-log-space": "false"}))
+    want = {"averageDepth": 2.0, "categoricalCount": 0, "constantCount": 0, "featureCount": 2, "gaussianCount": 0, "histogramCount": 2,
+            "innerCount": 1, "leafCount": 2, "maxDepth": 2, "medianDepth": 1.5, "minDepth": 2, "productCount": 1, "sumCount": 0}
+    assert {k_: st[k_] for k_ in want} == want
+    assert '"averageDepth":2.0,' in open(out).read()
+    # log space has no final log operation: every depth is one less
+    st = stats(compile_spn(native, Product(children=hists), "int32", **stats_opts))
+    assert (st["minDepth"], st["maxDepth"], st["averageDepth"]) == (1, 1, 1.0)
+
+    # The region graph shares every node among 8 or 64 parents: 1e10 root-to-leaf paths, counted by recurrence.
+    from spnc import synthetic as syn
+    st = stats(compile_spn(native, syn.c4_spn(), "float32", **stats_opts))
+    # 10 repetitions of: 16 leaf regions of 4 products of two leaves; 8 regions of 8 sums over 4 x 4 products; 7 regions of
+    # 8 sums over 8 x 8 products; and the root sum over the 80 root-region sums.
+    terms = 10 * (8 * 8 * 16 + 7 * 8 * 64) + 80
+    assert st["gaussianCount"] == 10 * 16 * 4 * 2 and st["constantCount"] == terms
+    assert st["sumCount"] == 10 * (8 * 8 * 15 + 7 * 8 * 63) + 79
+    assert st["productCount"] == terms + 10 * (8 * 16 + 7 * 64) + 10 * 16 * 4
+    assert st["hip"]["depthsExact"] is False and st["minDepth"] < st["averageDepth"] < st["maxDepth"]
+    with pytest.raises(RuntimeError, match="cannot write graph statistics"):
+        compile_query(native, os.path.join(GOLDEN, "NIPS5.bin"), **{"collect-graph-stats": "true", "graph-stats-file": str(tmp_path / "no" / "dir.json")})
+
+
+def test_table_index_is_compared_in_a_wide_type(native):
+    """A table as long as (or longer than) the feature type's range must not wrap the bound of the index clamp."""
+    from spnc.structure import Categorical, Product
+    for dtype, entries in (("uint8", 256), ("uint8", 300), ("uint16", 65536), ("uint64", 5)):
+        p = np.full(entries, 1.0 / entries)
+        k = compile_spn(native, Product(children=[Categorical(p=list(p), scope=0), Categorical(p=[0.5, 0.5], scope=1)]), dtype,
+                        **{"hip-kernel": "jit"})
+        src = k.source()
+        os.remove(k.fileName())
+        assert "(feat_t)" + str(entries) not in src
+        wide = "(unsigned long long)x[0] < %dull" % entries if dtype == "uint64" else "(unsigned)x[0] < %du" % entries
+        assert wide in src
+
+
+def test_damaged_kernel_files_are_rejected(native, tmp_path):
+    """Every field of a kernel file is checked on the host before anything could reach a launch."""
+    from spnc import synthetic as syn
+    import struct
+    for opts in ({}, {"hip-kernel": "interpreter"}):
+        k = compile_spn(native, syn.c4_spn() if opts else syn.c1_spn(), "float32" if opts else "int32", **opts)
+        blob = open(k.fileName(), "rb").read()
+        os.remove(k.fileName())
+        bad = tmp_path / "bad.hipk"
+        bad.write_bytes(blob[: len(blob) // 2])
+        with pytest.raises(RuntimeError, match="truncated kernel file|damaged|malformed"):
+            native.Kernel(str(bad))
+        bad.write_bytes(blob + b"\0\0\0\0")
+        with pytest.raises(RuntimeError, match="trailing bytes"):
+            native.Kernel(str(bad))
+        name_len = struct.unpack_from("<Q", blob, 8)[0]
+        fields = 8 + 8 + name_len     # batchSize, numFeatures, bytesPerFeature, bytesPerResult, featureType
+        for index, value, what in ((1, 0, "feature count"), (2, 3, "feature width"), (3, 0, "result width"), (4, 77, "feature type")):
+            b = bytearray(blob)
+            struct.pack_into("<I", b, fields + 4 * index, value)
+            bad.write_bytes(bytes(b))
+            with pytest.raises(RuntimeError, match=what):
+                native.Kernel(str(bad))
+    # interpreter programs: a slot number out of range, a broken length word and a bad opcode anywhere in the stream
+    words = np.frombuffer(blob, dtype="<u4", offset=len(blob) % 4)
+    code_words = k.info()["num_nodes"]  # just a lower bound on the stream length, for the search below
+    assert code_words > 1000
+    tail = len(blob) - 5 * 4 - 8 - 4 * 4 * 32 - 8   # somewhere inside the weights and slot lists: find the END instruction instead
+    # the stream ends with [2][OP_END][slot]; the five u32 trailer fields and the staged list follow it
+    b = bytearray(blob)
+    hits = [i for i in range(len(b) - 12, 0, -4) if struct.unpack_from("<II", b, i) == (2, 0) or struct.unpack_from("<II", b, i)[0:2] == (2, 0x80)]
+    assert hits
+    end_at = hits[0]
+    struct.pack_into("<I", b, end_at + 8, 1 << 19)
+    bad.write_bytes(bytes(b))
+    with pytest.raises(RuntimeError, match="malformed interpreter program \\(slot number"):
+        native.Kernel(str(bad))
+    b = bytearray(blob)
+    struct.pack_into("<I", b, end_at + 4, 0x7f)
+    bad.write_bytes(bytes(b))
+    with pytest.raises(RuntimeError, match="malformed interpreter program"):
+        native.Kernel(str(bad))
+    b = bytearray(blob)
+    struct.pack_into("<I", b, end_at, 3)
+    bad.write_bytes(bytes(b))
+    with pytest.raises(RuntimeError, match="malformed interpreter program"):
+        native.Kernel(str(bad))
+
+
+def test_execute_checks_the_input_type_not_only_its_width(native):
+    from spnc import synthetic as syn
+    k = compile_spn(native, syn.c2_spn(), "float32")
     os.remove(k.fileName())
+    assert k.info()["feature_is_float"] == 1 and k.info()["support_marginal"] == 0
+    with pytest.raises(RuntimeError, match="does not match the kernel's feature type float32"):
+        k.execute(4, np.zeros((4, 16), dtype=np.int32))
+    with pytest.raises(RuntimeError, match="does not match the kernel's feature type float32"):
+        k.execute(4, np.zeros((4, 16), dtype=np.float64))
+    k = compile_spn(native, syn.c1_spn(), "int32")
+    os.remove(k.fileName())
+    assert k.info()["feature_is_float"] == 0
+    with pytest.raises(RuntimeError, match="does not match the kernel's feature type int32"):
+        k.execute(4, np.zeros((4, 6), dtype=np.float32))
+
+
+def test_host_feature_queries(native):
+    flags = open("/proc/cpuinfo").read()
+    C = native.SPNCompiler
+    assert C.isFeatureAvailable("AVX2") == (" avx2" in flags) and C.isFeatureAvailable("vectorize") == (C.isFeatureAvailable("AVX") or C.isFeatureAvailable("Neon"))
+    assert C.isFeatureAvailable("no-such-feature") is False
 
 
 def _bad(native, tmp_path, match, **kw):
@@ -235,7 +373,7 @@ def test_grouped_table_layout(native):
     """Table-heavy graphs: tables read with the same index share blocks of four columns, indices are packed four to a
     register, and the block size goes to 1024; small graphs and the option switch keep plain tables."""
     from spnc import synthetic as syn
-    k = compile_spn(native, syn.c3_spn(), "int32", marginal=False)
+    k = compile_spn(native, syn.c3_deep_spn(), "int32", marginal=False)
     src = k.source()
     os.remove(k.fileName())
     reads = src.count("*>(reinterpret_cast<const char*>(tab + ")
@@ -243,7 +381,7 @@ def test_grouped_table_layout(native):
     assert "const unsigned P24 = " in src and "#define SPN_BLOCK 1024" in src and "__launch_bounds__(SPN_BLOCK, 1)" in src
     pool = int(re.search(r"#define SPN_NTAB (\d+)", src).group(1))
     assert pool % 4 == 0 and pool * 4 <= 80 * 1024
-    k = compile_spn(native, syn.c3_spn(), "int32", marginal=False, **{"hip-grouped-tables": "false"})
+    k = compile_spn(native, syn.c3_deep_spn(), "int32", marginal=False, **{"hip-grouped-tables": "false"})
     src = k.source()
     os.remove(k.fileName())
     assert "spn_r4 q" not in src and "v_bfe_u32" not in src and "#define SPN_BLOCK 256" in src and src.count("= tab[") == 1940
