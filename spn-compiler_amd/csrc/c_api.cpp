@@ -10,6 +10,9 @@
 #include "../../include/spnc_hip.h"
 #include "kernel.h"
 
+#include "interp_kernel.h"
+static_assert(SPNC_HIP_STATIC_SCRATCH_BYTES == spnc_hip::INTERP_SCRATCH_BYTES, "the header states the size of the scratch array");
+
 struct spnc_hip_kernel {
   std::unique_ptr<spnc_hip::Kernel> impl;
 };
@@ -87,6 +90,13 @@ int spnc_hip_execute_device(spnc_hip_kernel* k, size_t n, const void* d_in, void
   return guarded([&] {
     if (!k) throw std::runtime_error("null kernel");
     k->impl->executeDevice(n, d_in, d_out, static_cast<hipStream_t>(stream));
+  });
+}
+
+int spnc_hip_execute_device_static(spnc_hip_kernel* k, size_t n, const void* d_in, void* d_out, void* stream) {
+  return guarded([&] {
+    if (!k) throw std::runtime_error("null kernel");
+    k->impl->executeDeviceStatic(n, d_in, d_out, static_cast<hipStream_t>(stream));
   });
 }
 

@@ -31,6 +31,11 @@ struct InterpLaunch {
 hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain, int mode, unsigned grid, size_t ldsBytes,
                              hipStream_t stream);
 
+// Device memory of the allocation-free entry point: one array per device inside the library's code object, held
+// from library load to process end. Returns its address on the current device and its size.
+constexpr size_t INTERP_SCRATCH_BYTES = size_t(64) << 20;
+hipError_t interpreterScratch(void** base, size_t* bytes);
+
 // Largest dynamic LDS size a block of the interpreter may request on the current device.
 hipError_t interpreterMaxLds(bool f64, bool log2Domain, size_t* bytes);
 

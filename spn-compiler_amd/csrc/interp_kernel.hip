@@ -14,6 +14,8 @@
 // mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:306-374 and :440-529.
 #include "interp_kernel.h"
 
+#include <mutex>
+
 #include "interp_program.h"
 #include "spn_graph.h"
 
@@ -1028,6 +1030,31 @@ const void* pick(bool f64, bool log2Domain, int mode, bool staged) {
 }
 
 }  // namespace
+
+namespace {
+// Scratch memory of the allocation-free entry point. The name is a host-side handle only: device code and every
+// runtime call get the address that hipGetSymbolAddress returns for the current device.
+static __device__ __align__(256) unsigned char scratch[INTERP_SCRATCH_BYTES];
+std::mutex scratchMutex;
+void* scratchAddress[64] = {};
+}  // namespace
+
+hipError_t interpreterScratch(void** base, size_t* bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(scratchMutex);
+  if (!scratchAddress[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    scratchAddress[dev] = p;
+  }
+  *base = scratchAddress[dev];
+  *bytes = INTERP_SCRATCH_BYTES;
+  return hipSuccess;
+}
 
 hipError_t interpreterMaxLds(bool f64, bool log2Domain, size_t* bytes) {
   int dev = 0, maxLds = 0;

@@ -4,6 +4,7 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -380,7 +381,9 @@ void Kernel::ensureDevice() {
   deviceReady_ = true;
 }
 
-void Kernel::prepareDevice() {
+// What the launcher needs to know about the device and the kernel's footprint on it. Allocates nothing.
+void Kernel::queryDevice() {
+  if (deviceKnown_) return;
   int count = 0;
   if (hipGetDeviceCount(&count) != hipSuccess || count == 0) fatal("RUNTIME ERROR: no HIP device available");
   hipCheck(hipGetDevice(&device_), "hipGetDevice");
@@ -389,13 +392,7 @@ void Kernel::prepareDevice() {
   if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     fatal(std::string("RUNTIME ERROR: kernels are built for gfx950, device is ") + prop.gcnArchName);
   numCUs_ = prop.multiProcessorCount;
-  if (kind_ == SPNC_HIP_KERNEL_JIT) {
-    hipCheck(hipModuleLoadData(&module_, codeObject_.data()), "hipModuleLoadData");
-    hipCheck(hipModuleGetFunction(&function_, module_, entry_.c_str()), "hipModuleGetFunction");
-    int nb = 0;
-    hipCheck(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&nb, function_, int(blockSize_), 0), "occupancy query");
-    blocksPerCU_ = std::max(1, nb);
-  } else {
+  if (kind_ == SPNC_HIP_KERNEL_INTERPRETER) {
     const size_t rb = prog_.f64 ? 8 : 4;
     // Value slots in LDS: as many as the program needs, capped so that two blocks fit a CU.
     int ldsPerCU = 0;
@@ -420,29 +417,55 @@ void Kernel::prepareDevice() {
     hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, interpMode_, prog_.featureMode == FEAT_STAGED, ldsBytes_, &nb), "occupancy query");
     blocksPerCU_ = std::max(1, nb);
     if (gridPolicy_ > 0) blocksPerCU_ = std::min(blocksPerCU_, gridPolicy_);  // "hip-blocks-per-cu": fewer than fit
-    // The kernel touches the cache lines that follow an instruction's weights, so the stream is padded past its end.
-    hipCheck(hipMalloc(&dCode_, prog_.code.size() * 4 + 512), "hipMalloc(program)");
-    hipCheck(hipMemset(dCode_, 0, prog_.code.size() * 4 + 512), "program padding");
-    hipCheck(hipMemcpy(dCode_, prog_.code.data(), prog_.code.size() * 4, hipMemcpyHostToDevice), "program upload");
-    if (!prog_.tables.empty()) {
-      hipCheck(hipMalloc(&dTables_, prog_.tables.size() * rb), "hipMalloc(tables)");
-      if (prog_.f64) {
-        hipCheck(hipMemcpy(dTables_, prog_.tables.data(), prog_.tables.size() * 8, hipMemcpyHostToDevice), "table upload");
-      } else {
-        std::vector<float> t(prog_.tables.begin(), prog_.tables.end());
-        hipCheck(hipMemcpy(dTables_, t.data(), t.size() * 4, hipMemcpyHostToDevice), "table upload");
-      }
+  }
+  deviceKnown_ = true;
+}
+
+// The interpreter's constant operands as the device holds them: the instruction stream followed by 512 zero bytes
+// (the kernel touches the cache lines that follow an instruction's weights and prefetches one head past the end),
+// the table pool in the compute type, and four words per staged feature.
+void Kernel::buildImages() {
+  if (!codeImage_.empty()) return;
+  codeImage_.assign(prog_.code.begin(), prog_.code.end());
+  codeImage_.resize(prog_.code.size() + 128, 0u);
+  const size_t rb = prog_.f64 ? 8 : 4;
+  tableImage_.resize(prog_.tables.size() * rb);
+  if (prog_.f64) {
+    if (!prog_.tables.empty()) std::memcpy(tableImage_.data(), prog_.tables.data(), tableImage_.size());
+  } else {
+    for (size_t i = 0; i < prog_.tables.size(); ++i) {
+      const float v = float(prog_.tables[i]);
+      std::memcpy(tableImage_.data() + 4 * i, &v, 4);
     }
-    if (!prog_.staged.empty()) {
-      std::vector<uint32_t> st;
-      for (const auto& s : prog_.staged) {
-        st.push_back(s.column);
-        st.push_back(s.valueSlot);
-        st.push_back(s.indexSlot);
-        st.push_back(s.tableLen);
-      }
-      hipCheck(hipMalloc(&dStaged_, st.size() * 4), "hipMalloc(staged)");
-      hipCheck(hipMemcpy(dStaged_, st.data(), st.size() * 4, hipMemcpyHostToDevice), "staged upload");
+  }
+  for (const auto& sf : prog_.staged) {
+    stagedImage_.push_back(sf.column);
+    stagedImage_.push_back(sf.valueSlot);
+    stagedImage_.push_back(sf.indexSlot);
+    stagedImage_.push_back(sf.tableLen);
+  }
+}
+
+void Kernel::prepareDevice() {
+  queryDevice();
+  if (kind_ == SPNC_HIP_KERNEL_JIT) {
+    hipCheck(hipModuleLoadData(&module_, codeObject_.data()), "hipModuleLoadData");
+    hipCheck(hipModuleGetFunction(&function_, module_, entry_.c_str()), "hipModuleGetFunction");
+    int nb = 0;
+    hipCheck(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&nb, function_, int(blockSize_), 0), "occupancy query");
+    blocksPerCU_ = std::max(1, nb);
+  } else {
+    const size_t rb = prog_.f64 ? 8 : 4;
+    buildImages();
+    hipCheck(hipMalloc(&dCode_, codeImage_.size() * 4), "hipMalloc(program)");
+    hipCheck(hipMemcpy(dCode_, codeImage_.data(), codeImage_.size() * 4, hipMemcpyHostToDevice), "program upload");
+    if (!tableImage_.empty()) {
+      hipCheck(hipMalloc(&dTables_, tableImage_.size()), "hipMalloc(tables)");
+      hipCheck(hipMemcpy(dTables_, tableImage_.data(), tableImage_.size(), hipMemcpyHostToDevice), "table upload");
+    }
+    if (!stagedImage_.empty()) {
+      hipCheck(hipMalloc(&dStaged_, stagedImage_.size() * 4), "hipMalloc(staged)");
+      hipCheck(hipMemcpy(dStaged_, stagedImage_.data(), stagedImage_.size() * 4, hipMemcpyHostToDevice), "staged upload");
     }
     const size_t lanes = size_t(numCUs_) * blocksPerCU_ * INTERP_BLOCK;
     spillBytes_ = size_t(prog_.numSlots - ldsSlots_) * lanes * rb;
@@ -493,31 +516,89 @@ void Kernel::launch(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
     void* args[] = {(void*)&dIn, (void*)&dOut, (void*)&n64};
     hipCheck(hipModuleLaunchKernel(function_, grid, 1, 1, blockSize_, 1, 1, 0, stream, args, nullptr), "kernel launch");
   } else {
-    const size_t tiles = (n + INTERP_BLOCK - 1) / INTERP_BLOCK;
-    const unsigned grid = unsigned(std::min<size_t>(tiles, size_t(numCUs_) * blocksPerCU_));
-    InterpLaunch a;
-    a.code = dCode_;
-    a.in = dIn;
-    a.out = dOut;
-    a.n = n;
-    a.tables = dTables_;
-    a.spill = dSpill_;
-    a.staged = dStaged_;
-    a.numStaged = uint32_t(prog_.staged.size());
-    a.numFeatures = numFeatures_;
-    a.featureType = featureType_;
-    a.featureMode = prog_.featureMode;
-    a.ldsSlots = ldsSlots_;
-    a.spillSlots = prog_.numSlots - ldsSlots_;
-    a.marginal = marginal_ ? 1u : 0u;
-    hipCheck(launchInterpreter(a, prog_.f64, prog_.log2Domain, interpMode_, grid, ldsBytes_, stream), "interpreter launch");
+    launchProgram(n, dIn, dOut, dCode_, dTables_, dStaged_, dSpill_, size_t(numCUs_) * blocksPerCU_, stream);
   }
+}
+
+void Kernel::launchProgram(size_t n, const void* dIn, void* dOut, const uint32_t* code, const void* tables, const uint32_t* staged,
+                           void* spill, size_t maxBlocks, hipStream_t stream) {
+  const size_t tiles = (n + INTERP_BLOCK - 1) / INTERP_BLOCK;
+  const unsigned grid = unsigned(std::min<size_t>(tiles, maxBlocks));
+  InterpLaunch a;
+  a.code = code;
+  a.in = dIn;
+  a.out = dOut;
+  a.n = n;
+  a.tables = tables;
+  a.spill = spill;
+  a.staged = staged;
+  a.numStaged = uint32_t(prog_.staged.size());
+  a.numFeatures = numFeatures_;
+  a.featureType = featureType_;
+  a.featureMode = prog_.featureMode;
+  a.ldsSlots = ldsSlots_;
+  a.spillSlots = prog_.numSlots - ldsSlots_;
+  a.marginal = marginal_ ? 1u : 0u;
+  hipCheck(launchInterpreter(a, prog_.f64, prog_.log2Domain, interpMode_, grid, ldsBytes_, stream), "interpreter launch");
 }
 
 void Kernel::executeDevice(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
   std::lock_guard<std::mutex> lock(mu_);
   ensureDevice();
   launch(n, dIn, dOut, stream);
+}
+
+namespace {
+std::mutex g_scratchMutex;
+uint64_t g_scratchOwner[64] = {};   // per device: id of the kernel whose program the scratch array holds (0 = none)
+std::atomic<uint64_t> g_nextKernelId{1};
+size_t roundUp256(size_t v) { return (v + 255) / 256 * 256; }
+}  // namespace
+
+// The launch of executeDevice() for interpreter kernels with every device buffer the kernel needs besides the
+// caller's input and output carved out of the library's fixed scratch array: program, tables, staged-feature
+// descriptors, then the spill tier, as many blocks' worth as fit (the grid shrinks to that). Calls no allocator.
+void Kernel::executeDeviceStatic(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(mu_);
+  if (kind_ != SPNC_HIP_KERNEL_INTERPRETER)
+    fatal("RUNTIME ERROR: the allocation-free entry point runs interpreter kernels (compile with hip-kernel=interpreter); "
+          "a straight-line kernel has no scratch memory, but loading its code object allocates");
+  queryDevice();
+  if (n == 0) return;
+  if (reinterpret_cast<uintptr_t>(dIn) % inputAlign_ != 0)
+    fatal("RUNTIME ERROR: input pointer must be aligned to " + std::to_string(inputAlign_) + " bytes");
+  if (reinterpret_cast<uintptr_t>(dOut) % bytesPerResult_ != 0) fatal("RUNTIME ERROR: output pointer is misaligned");
+  buildImages();
+  if (!kernelId_) kernelId_ = g_nextKernelId.fetch_add(1);
+  void* base = nullptr;
+  size_t capacity = 0;
+  hipCheck(interpreterScratch(&base, &capacity), "hipGetSymbolAddress(scratch)");
+  const size_t rb = prog_.f64 ? 8 : 4;
+  const size_t codeAt = 0, tablesAt = roundUp256(codeImage_.size() * 4), stagedAt = tablesAt + roundUp256(tableImage_.size()),
+               spillAt = stagedAt + roundUp256(stagedImage_.size() * 4);
+  const size_t spillPerBlock = size_t(prog_.numSlots - ldsSlots_) * INTERP_BLOCK * rb;
+  if (spillAt + spillPerBlock > capacity)
+    fatal("RUNTIME ERROR: the program needs " + std::to_string(spillAt + spillPerBlock) + " bytes of scratch memory (program, tables and one "
+          "block's spilled values), the allocation-free entry point has " + std::to_string(capacity) + "; use spnc_hip_execute_device");
+  size_t maxBlocks = size_t(numCUs_) * blocksPerCU_;
+  if (spillPerBlock) maxBlocks = std::min(maxBlocks, (capacity - spillAt) / spillPerBlock);
+  char* p = static_cast<char*>(base);
+  {
+    std::lock_guard<std::mutex> scratchLock(g_scratchMutex);
+    if (device_ < 0 || device_ >= 64) fatal("RUNTIME ERROR: device ordinal out of range");
+    if (g_scratchOwner[device_] != kernelId_) {
+      g_scratchOwner[device_] = 0;  // stays "nobody's" if an upload fails half way
+      hipCheck(hipMemcpyAsync(p + codeAt, codeImage_.data(), codeImage_.size() * 4, hipMemcpyHostToDevice, stream), "program upload");
+      if (!tableImage_.empty())
+        hipCheck(hipMemcpyAsync(p + tablesAt, tableImage_.data(), tableImage_.size(), hipMemcpyHostToDevice, stream), "table upload");
+      if (!stagedImage_.empty())
+        hipCheck(hipMemcpyAsync(p + stagedAt, stagedImage_.data(), stagedImage_.size() * 4, hipMemcpyHostToDevice, stream), "staged upload");
+      g_scratchOwner[device_] = kernelId_;
+    }
+  }
+  launchProgram(n, dIn, dOut, reinterpret_cast<const uint32_t*>(p + codeAt), tableImage_.empty() ? nullptr : p + tablesAt,
+                stagedImage_.empty() ? nullptr : reinterpret_cast<const uint32_t*>(p + stagedAt), spillPerBlock ? p + spillAt : nullptr,
+                maxBlocks, stream);
 }
 
 void Kernel::ensureStaging(size_t rows) {

@@ -37,12 +37,19 @@ class Kernel {
   void execute(size_t n, const void* in, void* out);
   // Device buffers; enqueues on `stream` and returns.
   void executeDevice(size_t n, const void* dIn, void* dOut, hipStream_t stream);
+  // The same for interpreter kernels without any allocation: the kernel's device buffers come out of the library's
+  // fixed scratch array (interp_kernel.h). Calls that overlap on one device race on that array.
+  void executeDeviceStatic(size_t n, const void* dIn, void* dOut, hipStream_t stream);
 
  private:
   Kernel() = default;
   void save(const std::string& path) const;
   void ensureDevice();
+  void queryDevice();
+  void buildImages();
   void prepareDevice();
+  void launchProgram(size_t n, const void* dIn, void* dOut, const uint32_t* code, const void* tables, const uint32_t* staged, void* spill,
+                     size_t maxBlocks, hipStream_t stream);
   void releaseDevice();
   void ensureStaging(size_t rows);
   void launch(size_t n, const void* dIn, void* dOut, hipStream_t stream);
@@ -66,7 +73,11 @@ class Kernel {
 
   // ---- device state, created on first execute ----
   std::mutex mu_;
-  bool deviceReady_ = false;
+  bool deviceReady_ = false;   // module loaded / device buffers allocated
+  bool deviceKnown_ = false;   // device facts and the kernel's launch shape queried
+  uint64_t kernelId_ = 0;      // tag of this kernel's program in the shared scratch array
+  std::vector<uint32_t> codeImage_, stagedImage_;  // what the device holds of the program (built once)
+  std::vector<char> tableImage_;
   int device_ = 0;
   int numCUs_ = 0;
   hipModule_t module_ = nullptr;

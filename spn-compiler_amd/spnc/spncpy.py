@@ -67,6 +67,7 @@ def _load():
     lib.spnc_hip_kernel_info.argtypes = [vp, ctypes.POINTER(_Info)]
     lib.spnc_hip_execute.argtypes = [vp, sz, vp, vp]
     lib.spnc_hip_execute_device.argtypes = [vp, sz, vp, vp, vp]
+    lib.spnc_hip_execute_device_static.argtypes = [vp, sz, vp, vp, vp]
     lib.spnc_hip_kernel_source.argtypes = [vp, ctypes.POINTER(cp), ctypes.POINTER(sz)]
     lib.spnc_hip_destroy.argtypes = [vp]
     lib.spnc_hip_destroy.restype = None
@@ -166,6 +167,13 @@ class Kernel:
         """Device pointers in/out; enqueues on ``stream`` (a hipStream_t as integer) without waiting."""
         _check(_load().spnc_hip_execute_device(self._handle, num_elements, ctypes.c_void_p(input_ptr),
                                                ctypes.c_void_p(output_ptr), ctypes.c_void_p(stream)))
+
+
+    def execute_device_static(self, num_elements, input_ptr, output_ptr, stream=0):
+        """``execute_device`` for interpreter kernels without any allocation: the kernel's device buffers come out of
+        a fixed scratch array inside the library. Calls that overlap on one GPU race on that array."""
+        _check(_load().spnc_hip_execute_device_static(self._handle, num_elements, ctypes.c_void_p(input_ptr),
+                                                      ctypes.c_void_p(output_ptr), ctypes.c_void_p(stream)))
 
 
 class SPNCompiler:

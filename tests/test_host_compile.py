@@ -18,7 +18,7 @@ MODELS = ["nltcs", "plants", "fashion_mnist"]
 def test_library_exports_every_declared_symbol(native):
     header = open(os.path.join(ROOT, "include", "spnc_hip.h")).read()
     declared = re.findall(r"SPNC_HIP_API[^;(]*?\b(spnc_hip_\w+)\s*\(", header)
-    assert len(declared) == 9
+    assert len(declared) == 10
     lib = ctypes.CDLL(native.library_path())
     for name in declared:
         assert hasattr(lib, name), name
