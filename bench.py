@@ -39,11 +39,11 @@ def make_inputs(name, cfg, n, torch, device):
     """Synthetic inputs of the configuration's shape and distribution, generated on the device."""
     from spnc import synthetic as syn
     g = torch.Generator(device=device)
-    g.manual_seed({"c1": 1, "c2": 102, "c3": 103, "c4": 104, "c5": 102}[name])
+    g.manual_seed({"c1": 1, "c2": 102, "c3": 103, "c3_deep": 103, "c4": 104, "c5": 102}[name])
     F = cfg["features"]
     if name == "c1":
         return torch.randint(0, 3, (n, F), generator=g, device=device, dtype=torch.int32)
-    if name == "c3":
+    if name in ("c3", "c3_deep"):
         doms = torch.tensor([d for _, d in syn.c3_domains()], device=device, dtype=torch.float32)
         u = torch.rand((n, F), generator=g, device=device)
         return torch.minimum((u * doms).floor(), doms - 1).to(torch.int32)
@@ -194,7 +194,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "c5_f64"])
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c3_deep", "c4", "c5", "c5_f64"])
     ap.add_argument("--n", type=int, default=0, help="override the number of samples")
     ap.add_argument("--no-others", action="store_true", help="measure only the selected configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")

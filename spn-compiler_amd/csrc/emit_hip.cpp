@@ -684,6 +684,31 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   }
   js.libraryMath = !e.log2Dom;
   js.doubleConstants = e.f64;
+  // Wide rows of 32-bit integer features read only by table leaves: a lane that fetches its own row touches 64 cache
+  // lines per load instruction of its wavefront, which keeps the memory pipeline at half the bandwidth of a plain copy
+  // (measured on 400-byte rows: 1.0 ms for 3.4 GB against 0.53 ms). Instead every wavefront copies the 64 rows of its
+  // tile, which are contiguous in memory, with fully coalesced 16-byte loads, packs each loaded vector of four values
+  // into four bytes (an index above 255 is out of every table's range anyway), writes the packed tile into its own LDS
+  // buffer and lets every lane read its row back: F/4 LDS writes and F/4 reads per sample, and memory at copy speed
+  // with as few as two wavefronts per SIMD.
+  bool waveTile = false;
+  unsigned waveStride = 0;  // dwords per packed row in LDS: odd, so that the 64 lanes' reads fall into distinct banks
+  {
+    bool eligible = e.vectorRows && !g.ftype.isFloat && eb == 4 && F % 4 == 0 && U == 1 && rowBytes >= 128;
+    for (uint32_t f = 0; f < F && eligible; ++f)
+      if (e.featGauss[f] || e.featTableLen[f] > 255) eligible = false;
+    if (eligible && o.waveTranspose == 1) {  // measured on the 100-feature discrete graphs: no gain yet beside unpacked indices (0.79 against 0.78 ms), so only on request
+      waveStride = (F / 4) | 1u;
+      const size_t tables = js.tablesInLds ? size_t(js.tableEntries) * realBytes : 0;
+      unsigned block = o.blockSize ? unsigned(o.blockSize) : 512u;
+      while (!o.blockSize && block > 64 && tables + size_t(block / 64) * 64 * waveStride * 4 > 150 * 1024) block /= 2;
+      if (tables + size_t(block / 64) * 64 * waveStride * 4 <= 150 * 1024) {
+        waveTile = true;
+        js.blockSize = block;
+      }
+    }
+  }
+  js.waveTransposedInput = waveTile;
 
   std::ostringstream s;
   s << "// generated by spnc-hip for SPN '" << g.name << "': " << g.nodes.size() << " nodes, " << F << " features\n";
@@ -816,7 +841,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   unsigned tableFeatures = 0;
   for (uint32_t f = 0; f < F; ++f) tableFeatures += e.featTableLen[f] ? 1 : 0;
   int minBlocks = o.minBlocksPerCU;
-  if (minBlocks == 0 && js.blockSize == 1024) minBlocks = 1;
+  if (minBlocks == 0 && (js.blockSize == 1024 || waveTile)) minBlocks = 1;
   if (minBlocks == 0 && js.tablesInLds && ldsTables > 40 * 1024 && ldsTables <= 80 * 1024 && tableFeatures <= 136) minBlocks = 2;
   s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK" << (minBlocks > 0 ? ", " + std::to_string(minBlocks) : std::string()) << ") " << js.entry
     << "(const feat_t* __restrict__ in, real_t* __restrict__ out, unsigned long long n) {\n";
@@ -843,12 +868,19 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   // than to the VALU bound (about 6.4e12 B/s against 6e13 lane-operations/s on MI355X).
   const double tHbm = double(rowBytes + realBytes) / 6.4e12, tValu = double(g.stats.issueSlotsMin()) / 6.0e13;
   const bool wantStaged = o.gpuSharedMem < 0 ? tHbm > 0.5 * tValu : o.gpuSharedMem == 1;
-  const bool staged = wantStaged && e.vectorRows && tileBytes % 16 == 0 && tileBytes + ldsTables <= 64 * 1024;
+  const bool staged = !waveTile && wantStaged && e.vectorRows && tileBytes % 16 == 0 && tileBytes + ldsTables <= 64 * 1024;
   js.stagedInput = staged;
   // Blocks with next to no set-up take one tile each; blocks that stage tables stay resident.
   js.oneTilePerBlock = js.tableEntries <= 256;
-  if (staged) js.inputAlign = 16;
+  if (staged || waveTile) js.inputAlign = 16;
+  if (waveTile) js.oneTilePerBlock = false;
   s << "  const unsigned long long tile = (unsigned long long)SPN_BLOCK * SPN_U;\n";
+  if (waveTile)
+    s << "  typedef unsigned int spn_v4 __attribute__((ext_vector_type(4)));\n"
+         "  constexpr unsigned SPN_Q = SPN_F / 4, SPN_S = " << waveStride << ";   // packed dwords per row, and their stride in LDS\n"
+         "  __shared__ unsigned spn_rows[SPN_BLOCK / 64][64 * SPN_S];\n"
+         "  const unsigned lane = threadIdx.x & 63u;\n"
+         "  unsigned* mine = spn_rows[threadIdx.x >> 6];\n";
   if (staged)
     s << "  typedef unsigned int spn_v4 __attribute__((ext_vector_type(4)));\n"
          "  __shared__ __attribute__((aligned(16))) feat_t spn_tile[SPN_BLOCK * SPN_U * SPN_F];\n";
@@ -862,7 +894,37 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
       "          out[i] = spn_eval(x, tab);\n"
       "        }\n"
       "      }\n";
-  if (staged) {
+  if (waveTile) {
+    // Piece p = 64 j + lane of the tile (16 bytes, four features of row p / Q) goes to packed dword p of the tile; row r's
+    // packed dwords r Q .. r Q + Q - 1 sit at stride S. A wavefront's LDS operations complete in order and no other
+    // wavefront touches its buffer, so no barrier is needed.
+    s << "    const unsigned long long first = base + (threadIdx.x & ~63u);   // first row of this wavefront's 64\n"
+         "    feat_t x[SPN_F];\n"
+         "    unsigned long long i = first + lane;\n"
+         "    if (first + 64 <= n) {\n"
+         "      const spn_v4* src = reinterpret_cast<const spn_v4*>(in + first * SPN_F);\n"
+         "      spn_v4 r[SPN_Q];\n"
+         "#pragma unroll\n"
+         "      for (unsigned j = 0; j < SPN_Q; ++j) r[j] = SPN_LOAD_TILE(src + j * 64 + lane);\n"
+         "#pragma unroll\n"
+         "      for (unsigned j = 0; j < SPN_Q; ++j) {\n"
+         "        const unsigned a = r[j][0] < 255u ? r[j][0] : 255u, b = r[j][1] < 255u ? r[j][1] : 255u;\n"
+         "        const unsigned c = r[j][2] < 255u ? r[j][2] : 255u, d = r[j][3] < 255u ? r[j][3] : 255u;\n"
+         "        const unsigned p = j * 64 + lane;\n"
+         "        mine[p + p / SPN_Q * (SPN_S - SPN_Q)] = a | (b << 8) | (c << 16) | (d << 24);\n"
+         "      }\n"
+         "#pragma unroll\n"
+         "      for (unsigned c = 0; c < SPN_Q; ++c) {\n"
+         "        const unsigned q = mine[lane * SPN_S + c];\n"
+         "        x[4 * c] = q & 255u;\n        x[4 * c + 1] = (q >> 8) & 255u;\n        x[4 * c + 2] = (q >> 16) & 255u;\n        x[4 * c + 3] = q >> 24;\n"
+         "      }\n"
+         "    } else {\n"
+         "      // the batch's last, partial group of 64 rows: every lane fetches its own row (idle lanes the last one)\n"
+         "      spn_load_row(in, i < n ? i : n - 1, x);\n"
+         "    }\n"
+         "    const real_t value = spn_eval(x, tab);\n"
+         "    if (i < n) __builtin_nontemporal_store(value, out + i);\n";
+  } else if (staged) {
     s << "    if (base + tile <= n) {\n"
          "      const spn_v4* src = reinterpret_cast<const spn_v4*>(in + base * SPN_F);\n"
          "      spn_v4* dst = reinterpret_cast<spn_v4*>(spn_tile);\n"

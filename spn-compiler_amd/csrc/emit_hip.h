@@ -24,6 +24,7 @@ struct JitSource {
   bool libraryMath = false;   // calls ocml exp/log (natural-log domain, linear space)
   bool doubleConstants = false;  // computes in double: constants live in registers, not in instruction literals
   bool oneTilePerBlock = false;
+  bool waveTransposedInput = false;  // every wavefront copies its 64 rows with coalesced loads, packed to bytes, through its own LDS buffer
   bool stagedInput = false;   // rows reach the lanes through an LDS tile ("gpu-shared-mem")
 };
 

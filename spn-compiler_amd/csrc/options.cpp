@@ -92,6 +92,8 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       if (o.samplesPerLane < 0 || o.samplesPerLane > 16) throw std::runtime_error("hip-samples-per-lane must be in [0,16]");
     } else if (key == "hip-jit-max-ops") {
       o.jitMaxOps = parseInt(key, val);
+    } else if (key == "hip-wave-transpose") {
+      o.waveTranspose = parseBool(val) ? 1 : 0;
     } else if (key == "hip-nontemporal-loads") {
       o.nontemporalLoads = parseBool(val);
     } else if (key == "hip-eager-indices") {
@@ -141,8 +143,8 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       if (o.blocksPerCU < -1 || o.blocksPerCU > 64) throw std::runtime_error("hip-blocks-per-cu must be in [-1,64]");
     } else if (key == "hip-block-size") {
       o.blockSize = parseInt(key, val);
-      if (o.blockSize != 0 && o.blockSize != 64 && o.blockSize != 128 && o.blockSize != 256 && o.blockSize != 512 && o.blockSize != 1024)
-        throw std::runtime_error("hip-block-size must be 64, 128, 256, 512 or 1024");
+      if (o.blockSize < 0 || o.blockSize > 1024 || o.blockSize % 64 != 0)
+        throw std::runtime_error("hip-block-size must be a multiple of 64 up to 1024");
     } else if (ignoredKeys().count(key)) {
       // accepted for compatibility, no effect on the HIP target
     } else {

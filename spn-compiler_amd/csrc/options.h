@@ -50,6 +50,7 @@ struct CompileOptions {
   int interpLdsSlots = 0;                      // "hip-interp-lds-slots": upper bound on the value slots the launcher keeps in LDS (0 = automatic)
   int interpStagedLong = -1;                   // "hip-interp-staged-features": lds|spill (-1 = automatic): tier of the staged input features
   long interpLongRange = -1;                   // "hip-interp-long-range": values living longer than this many instructions go to the long-lived pool (-1 = automatic)
+  int waveTranspose = -1;                       // "hip-wave-transpose": rows of 32-bit integer features reach the lanes through a per-wave LDS transpose of packed bytes (1), not (0), decided per kernel (-1)
   int minBlocksPerCU = 0;                      // "hip-min-blocks-per-cu": register budget hint for the generated kernel (0 = none)
   int blocksPerCU = 0;                         // "hip-blocks-per-cu": 0 = resident blocks (persistent), -1 = one tile per block, n = n per CU
 };

@@ -175,7 +175,6 @@ def test_grouped_tables_on_the_discrete_configuration(native, variant, cfg):
     if cfg == "c3":   # products of up to fifty leaves: which layout the generator picks is its own business, the values count
         src = None
     assert src is None or ("v_bfe_u32" in src) == grouped and ("spn_r4*" in src) == (grouped and variant != "singles"), variant
-    assert src is None or ("#define SPN_BLOCK 1024" in src) == (grouped and variant != "block-256")
     got = run(k, X)
     m = oracle_model(spn, c["dtype"])
     if variant == "float64":
