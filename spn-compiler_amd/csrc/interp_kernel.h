@@ -7,6 +7,7 @@
 namespace spnc_hip {
 
 constexpr unsigned INTERP_BLOCK = 256;
+constexpr unsigned INTERP_FEATURE_REGISTERS = 32;  // features a float kernel can keep in registers (FEAT_REGISTER programs)
 
 struct InterpLaunch {
   const uint32_t* code;      // device: instruction stream
@@ -19,7 +20,7 @@ struct InterpLaunch {
   uint32_t numStaged;
   uint32_t numFeatures;
   uint32_t featureType;      // spnc_hip::FeatureType as integer
-  uint32_t featureMode;      // FEAT_STAGED / FEAT_DIRECT
+  uint32_t featureMode;      // FEAT_STAGED / FEAT_DIRECT / FEAT_REGISTER
   uint32_t ldsSlots;         // slots [0, ldsSlots) live in LDS, the rest in the spill tier
   uint32_t spillSlots;       // number of slots in the spill tier
   uint32_t marginal;         // NaN features marginalise Gaussian leaves
@@ -39,8 +40,8 @@ hipError_t interpreterScratch(void** base, size_t* bytes);
 // Largest dynamic LDS size a block of the interpreter may request on the current device.
 hipError_t interpreterMaxLds(bool f64, bool log2Domain, size_t* bytes);
 
-// Resident blocks per CU for a given dynamic LDS size. staged: the program stages its features (args.featureMode
-// == FEAT_STAGED at launch); float kernels are built once per feature mode.
-hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, bool staged, size_t ldsBytes, int* blocksPerCU);
+// Resident blocks per CU for a given dynamic LDS size. featureMode: the program's (args.featureMode at launch);
+// float kernels are built once per feature mode.
+hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, uint32_t featureMode, size_t ldsBytes, int* blocksPerCU);
 
 }  // namespace spnc_hip

@@ -111,12 +111,19 @@ void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures) {
   const std::vector<uint32_t>& c = p.code;
   const size_t RW = p.f64 ? 2 : 1;
   if (p.shortSlots > p.numSlots || p.numSlots > (1u << 20)) bad("slot counts", 0);
-  if (p.featureMode != FEAT_STAGED && p.featureMode != FEAT_DIRECT) bad("feature mode", 0);
+  if (p.featureMode != FEAT_STAGED && p.featureMode != FEAT_DIRECT && p.featureMode != FEAT_REGISTER) bad("feature mode", 0);
+  const bool inRegisters = p.featureMode == FEAT_REGISTER;
+  if (inRegisters && (p.f64 || p.staged.size() > 32)) bad("register features", 0);
   if (p.f64 && p.log2Domain) bad("compute type", 0);
   std::map<uint32_t, uint32_t> indexBound;  // staged index slot -> largest index it can hold
   std::set<uint32_t> valueSlots;
-  for (const auto& sf : p.staged) {
+  for (size_t k = 0; k < p.staged.size(); ++k) {
+    const auto& sf = p.staged[k];
     if (sf.column >= numFeatures) bad("staged column", 0);
+    if (inRegisters) {
+      if (sf.valueSlot != k || sf.indexSlot != NONE) bad("feature register", 0);
+      continue;
+    }
     if (sf.valueSlot != NONE && sf.valueSlot >= p.numSlots) bad("staged value slot", 0);
     if (sf.indexSlot != NONE && sf.indexSlot >= p.numSlots) bad("staged index slot", 0);
     if (sf.tableLen > (1u << 24)) bad("staged table length", 0);
@@ -124,7 +131,7 @@ void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures) {
     if (sf.indexSlot != NONE) indexBound[sf.indexSlot] = sf.tableLen + 1;
   }
   const bool staged = p.featureMode == FEAT_STAGED;
-  if (!staged && !p.staged.empty()) bad("staged features in a direct-feature program", 0);
+  if (!staged && !inRegisters && !p.staged.empty()) bad("staged features in a direct-feature program", 0);
   size_t pc = 0;
   for (;;) {
     if (pc + 1 >= c.size()) bad("stream ends inside an instruction", pc);
@@ -152,6 +159,10 @@ void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures) {
     };
     auto feature = [&](size_t at, uint32_t tier) {
       if (at >= end) bad("feature field outside its instruction", pc);
+      if (inRegisters) {
+        if (c[at] >= p.staged.size()) bad("feature register", at);
+        return;
+      }
       if (!staged) {
         if (c[at] >= numFeatures) bad("feature column", at);
         return;
@@ -185,7 +196,7 @@ void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures) {
             if (it == indexBound.end()) bad("table index slot", q);
             bound = it->second;
           } else {
-            if (c[q] >= numFeatures) bad("feature column", q);
+            if (inRegisters || c[q] >= numFeatures) bad("feature column", q);
             bound = c[q + 2] + 1;
           }
           if (size_t(c[q + 1]) + bound >= p.tables.size()) bad("table offset", q + 1);
@@ -307,11 +318,29 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
     stagedSlots += (featGauss[f] ? 1 : 0) + (featTableLen[f] ? 1 : 0);
   }
   p.featureMode = stagedSlots <= 48 ? FEAT_STAGED : FEAT_DIRECT;
+  {
+    // Float programs whose features (at most 32) all feed Gaussian leaves keep them in registers for the whole tile:
+    // no slot, no memory access per use. (Measured on the RAT-SPN configuration: the staged features, kept in the
+    // spill tier, were re-read 320 times per sample, 4 GiB per launch.)
+    bool tablesUsed = false;
+    uint32_t gaussFeatures = 0;
+    for (uint32_t f = 0; f < g.numFeatures; ++f) {
+      tablesUsed = tablesUsed || featTableLen[f] != 0;
+      gaussFeatures += featGauss[f] ? 1 : 0;
+    }
+    if (o.interpFeatureRegisters && !p.f64 && !tablesUsed && gaussFeatures > 0 && gaussFeatures <= 32) p.featureMode = FEAT_REGISTER;
+  }
   std::vector<uint32_t> valueSlotOf(g.numFeatures, NONE), indexSlotOf(g.numFeatures, NONE);
   constexpr uint32_t LONG_BIT = 0x80000000u;  // marks long-pool slot numbers until they are renumbered
   uint32_t nextSlot = 0, longCount = 0;
   auto stagedSlot = [&]() { return stagedLong ? (LONG_BIT | longCount++) : nextSlot++; };
-  if (p.featureMode == FEAT_STAGED) {
+  if (p.featureMode == FEAT_REGISTER) {
+    for (uint32_t f = 0; f < g.numFeatures; ++f) {
+      if (!featGauss[f]) continue;
+      valueSlotOf[f] = uint32_t(p.staged.size());  // the register number
+      p.staged.push_back(StagedFeature{f, valueSlotOf[f], NONE, 0});
+    }
+  } else if (p.featureMode == FEAT_STAGED) {
     for (uint32_t f = 0; f < g.numFeatures; ++f) {
       if (!featGauss[f] && !featTableLen[f]) continue;
       StagedFeature sf{f, NONE, NONE, featTableLen[f]};
@@ -648,6 +677,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       double coef = -std::log(leaf.stddev) + -0.5 * std::log(2 * M_PI);
       double den = -(1.0 / (2.0 * leaf.stddev * leaf.stddev));
       if (p.featureMode == FEAT_STAGED) slotWord(valueSlotOf[leaf.feature]);
+      else if (p.featureMode == FEAT_REGISTER) b.word(valueSlotOf[leaf.feature]);
       else b.word(leaf.feature);
       b.real(leaf.mean);
       b.real(coef / den);  // value = den * (d * d + coef / den): one multiply-add and one multiply, each with one constant
@@ -841,6 +871,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
           for (uint32_t list : {region.a[0], region.b[0]})
             for (uint32_t c : g.nodes[list].children) {
               if (stagedFeatures) slotWord(valueSlotOf[g.nodes[c].feature]);
+              else if (p.featureMode == FEAT_REGISTER) b.word(valueSlotOf[g.nodes[c].feature]);
               else b.word(g.nodes[c].feature);
             }
         };
@@ -986,7 +1017,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   std::ostringstream hdr;
   hdr << "; interpreter program for SPN '" << g.name << "': " << instrs.size() << " instructions, " << p.code.size() << " words, "
       << p.numSlots << " value slots (" << p.reservedSlots << " staged features, " << (p.numSlots - p.shortSlots) << " long-lived), compute " << (p.f64 ? "f64" : "f32")
-      << (p.log2Domain ? " log2-domain" : "") << ", features " << (p.featureMode == FEAT_STAGED ? "staged" : "direct") << "\n";
+      << (p.log2Domain ? " log2-domain" : "") << ", features " << (p.featureMode == FEAT_STAGED ? "staged" : (p.featureMode == FEAT_REGISTER ? "in registers" : "direct")) << "\n";
   p.listing = hdr.str() + b.txt.str();
   return p;
 }

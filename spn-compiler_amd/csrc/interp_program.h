@@ -58,11 +58,13 @@ enum InterpOp : uint32_t {
 enum FeatureMode : uint32_t {
   FEAT_STAGED = 0,  // converted once per tile into reserved slots (feat fields hold slot numbers)
   FEAT_DIRECT = 1,  // read from the input row at each leaf (feat fields hold column numbers)
+  FEAT_REGISTER = 2,  // converted once per tile into registers (feat fields hold register numbers; float programs whose
+                      // features, at most 32, feed Gaussian leaves only). The staged list gives each register's column.
 };
 
 struct StagedFeature {
   uint32_t column;
-  uint32_t valueSlot;  // slot of the value converted to the compute type, or UINT32_MAX
+  uint32_t valueSlot;  // slot of the value converted to the compute type (FEAT_REGISTER: the register number), or UINT32_MAX
   uint32_t indexSlot;  // slot of the clamped table index (raw u32 bits), or UINT32_MAX
   uint32_t tableLen;   // clamp bound L: indices >= L select the "impossible" entry, NaN selects L+1
 };

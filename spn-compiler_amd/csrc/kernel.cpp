@@ -414,7 +414,7 @@ void Kernel::queryDevice() {
     }
     ldsBytes_ = size_t(ldsSlots_) * INTERP_BLOCK * rb;
     int nb = 0;
-    hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, interpMode_, prog_.featureMode == FEAT_STAGED, ldsBytes_, &nb), "occupancy query");
+    hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, interpMode_, prog_.featureMode, ldsBytes_, &nb), "occupancy query");
     blocksPerCU_ = std::max(1, nb);
     if (gridPolicy_ > 0) blocksPerCU_ = std::min(blocksPerCU_, gridPolicy_);  // "hip-blocks-per-cu": fewer than fit
   }

@@ -79,6 +79,8 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       else throw std::runtime_error("Could not parse option value " + val + " for " + key);
     } else if (key == "hip-log2-domain") {
       o.log2Domain = parseBool(val);
+    } else if (key == "hip-interp-feature-registers") {
+      o.interpFeatureRegisters = parseBool(val);
     } else if (key == "hip-interp-leaf-regions") {
       o.interpLeafRegions = parseBool(val);
     } else if (key == "hip-interp-vector-blocks") {

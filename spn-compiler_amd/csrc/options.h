@@ -47,6 +47,7 @@ struct CompileOptions {
   bool interpVectorBlocks = true;              // "hip-interp-vector-blocks": results of a matrix-form outer sum occupy consecutive slots
   bool interpScaledVectors = true;             // "hip-interp-scaled-vectors": region vectors between matrix-form outer sums travel as scaled linear values
   bool interpMatrixCore = true;                // "hip-interp-matrix-core": float outer sums of eight sums run on the matrix cores
+  bool interpFeatureRegisters = true;          // "hip-interp-feature-registers": float programs over at most 32 Gaussian-only features keep them in registers
   int interpLdsSlots = 0;                      // "hip-interp-lds-slots": upper bound on the value slots the launcher keeps in LDS (0 = automatic)
   int interpStagedLong = -1;                   // "hip-interp-staged-features": lds|spill (-1 = automatic): tier of the staged input features
   long interpLongRange = -1;                   // "hip-interp-long-range": values living longer than this many instructions go to the long-lived pool (-1 = automatic)

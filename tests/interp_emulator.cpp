@@ -56,6 +56,12 @@ int main(int argc, char** argv) {
         if (s.valueSlot != UINT32_MAX) slot.at(s.valueSlot) = float(x[s.column]);
         if (s.indexSlot != UINT32_MAX) slot.at(s.indexSlot) = float(index(x[s.column], s.tableLen));
       }
+      // A feature field of an instruction that does not read staged slots: an input column, or the number of the
+      // register that holds one (the staged list names its column).
+      auto field = [&](uint32_t w) -> float {
+        if (p.featureMode == FEAT_REGISTER) return float(x[p.staged.at(w).column]);
+        return float(x[w]);
+      };
       size_t pc = 0, expectedEnd = 0;
       for (;;) {
         if (pc != expectedEnd) throw std::runtime_error("length word disagrees with the instruction before word " + std::to_string(pc));
@@ -82,7 +88,7 @@ int main(int argc, char** argv) {
           for (uint32_t j = 0; j < ns; ++j) acc += rd(c.at(q + j));
           q += ns;
           for (uint32_t j = 0; j < ng; ++j, q += 4) {
-            const float xv = p.featureMode == FEAT_STAGED ? rd(c.at(q)) : float(x[c.at(q)]);
+            const float xv = p.featureMode == FEAT_STAGED ? rd(c.at(q)) : field(c.at(q));
             const float d = xv - asFloat(c.at(q + 1));
             float v = (d * d + asFloat(c.at(q + 2))) * asFloat(c.at(q + 3));
             if (g.supportMarginal && xv != xv) v = 0;
@@ -118,7 +124,7 @@ int main(int argc, char** argv) {
             const uint32_t dst = c.at(q++);
             float acc = 0;
             for (uint32_t j = 0; j < G; ++j, q += 4) {
-              const float xv = p.featureMode == FEAT_STAGED ? rd(c.at(q)) : float(x[c.at(q)]);
+              const float xv = p.featureMode == FEAT_STAGED ? rd(c.at(q)) : field(c.at(q));
               const float d = xv - asFloat(c.at(q + 1));
               float v = (d * d + asFloat(c.at(q + 2))) * asFloat(c.at(q + 3));
               if (g.supportMarginal && xv != xv) v = 0;
@@ -247,7 +253,7 @@ int main(int argc, char** argv) {
               for (uint32_t j = 0; j < G; ++j) {
                 const size_t q = rec + (size_t(i) * G + j) * 3;
                 const uint32_t fw = c.at(feat + (i < na ? 0 : G) + j);
-                const float xv = stagedFeatures ? rd(fw) : float(x[fw]);
+                const float xv = stagedFeatures ? rd(fw) : field(fw);
                 const float d = xv - asFloat(c.at(q));
                 float v = (d * d + asFloat(c.at(q + 1))) * asFloat(c.at(q + 2));
                 if (g.supportMarginal && xv != xv) v = 0;

@@ -339,6 +339,8 @@ def test_generated_source_variants(native):
     k = compile_spn(native, syn.c4_spn(), "float32")
     src = k.source()
     assert k.info()["kernel_kind"] == 2 and "outersum(8 sums x 8x8 products)" in src
+    # 32 features, Gaussian leaves only: they live in registers, not in value slots
+    assert "(0 staged features," in src and "features in registers" in src
     # the 160 leaf regions are computed inside the outer sums above them, four at a time with the three 8x8 sums over
     # them: no product instructions and no 4x4 outer sums at all; 8x8 sums of their own remain above (10 root regions
     # of two and one more level below them)
@@ -354,7 +356,8 @@ def test_generated_source_variants(native):
     assert i["trans_min"] < i["sum_terms"] // 10 and i["flops_min"] < 2 * i["sum_terms"]
     os.remove(k.fileName())
     # the program builder honours the tier and pool-size options
-    pools = {"hip-interp-staged-features": "lds", "hip-interp-long-range": 8, "hip-interp-short-slots": 40, "hip-interp-leaf-regions": "false"}
+    pools = {"hip-interp-staged-features": "lds", "hip-interp-long-range": 8, "hip-interp-short-slots": 40, "hip-interp-leaf-regions": "false",
+             "hip-interp-feature-registers": "false"}
     k = compile_spn(native, syn.c4_spn(), "float32", **pools)
     src = k.source()
     os.remove(k.fileName())
