@@ -23,6 +23,18 @@ def build():
     return _SO
 
 
+def threads(set_to=None):
+    """OpenMP threads the evaluator runs on; ``set_to`` changes the number for later calls."""
+    if not os.path.isfile(_SO):
+        build()
+    lib = ctypes.CDLL(_SO)
+    lib.spn_oracle_threads.restype = ctypes.c_int
+    if set_to is not None:
+        lib.spn_oracle_set_threads.argtypes = [ctypes.c_int]
+        lib.spn_oracle_set_threads(int(set_to))
+    return lib.spn_oracle_threads()
+
+
 def ll_f32(model, X, marginal=True):
     """f32 log-likelihoods in the reference's operation order, evaluated by the C restatement."""
     if not os.path.isfile(_SO):

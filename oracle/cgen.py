@@ -107,6 +107,7 @@ def generate(model, marginal, batch_size=4096):
     src = f"""// generated CPU baseline kernel: reference operation order, f32 log-space
 #include <math.h>
 #include <stddef.h>
+#include <omp.h>
 #pragma omp declare simd notinbranch
 extern float expf(float);
 #pragma omp declare simd notinbranch
@@ -126,6 +127,9 @@ static void spn_chunk(const {ctype}* restrict in, float* restrict out, size_t n)
       out[i] = v{model.root};
   }}
 }}
+// Threads the chunk loop runs on (what a caller reports as "cores"), and a way to time one thread.
+int spn_cpu_threads(void) {{ return omp_get_max_threads(); }}
+void spn_cpu_set_threads(int n) {{ omp_set_num_threads(n); }}
 // Chunks of batch_size samples in parallel, like Executable::executeBatch.
 void spn_cpu_execute(const {ctype}* in, float* out, size_t n) {{
   const size_t bs = {batch_size};
@@ -161,10 +165,16 @@ def load(so_path, feature_dtype):
     lib.spn_cpu_execute.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
     lib.spn_cpu_execute.restype = None
 
+    lib.spn_cpu_threads.restype = ctypes.c_int
+    lib.spn_cpu_set_threads.argtypes = [ctypes.c_int]
+    lib.spn_cpu_set_threads.restype = None
+
     def run(X):
         X = np.ascontiguousarray(X, dtype=np.dtype(feature_dtype))
         out = np.empty(X.shape[0], dtype=np.float32)
         lib.spn_cpu_execute(X.ctypes.data, out.ctypes.data, X.shape[0])
         return out
 
+    run.threads = lib.spn_cpu_threads          # OpenMP threads the next call will use
+    run.set_threads = lib.spn_cpu_set_threads
     return run

@@ -21,6 +21,7 @@
  * execute/src/main.cpp:32-52, the NIPS5 / nltcs / plants golden outputs, FileCheck constants).
  */
 #include <math.h>
+#include <omp.h>
 #include <stdlib.h>
 #include <stddef.h>
 
@@ -57,6 +58,10 @@ static float tree(const float* t, int lo, int hi, int is_sum) {
   const float l = tree(t, lo, pivot, is_sum), r = tree(t, pivot, hi, is_sum);
   return is_sum ? logadd(l, r) : l + r;
 }
+
+/* Threads the sample loop runs on, and a way to time a single one (bench.py's cpu_baseline). */
+int spn_oracle_threads(void) { return omp_get_max_threads(); }
+void spn_oracle_set_threads(int n) { omp_set_num_threads(n); }
 
 /* in: [n, num_features] as double (integers exactly representable); out: [n] float. */
 int spn_oracle_f32(const spn_flat* s, const double* in, size_t n, int marginal, float* out) {

@@ -5,6 +5,8 @@
 
 #include <algorithm>
 #include <atomic>
+#include <condition_variable>
+#include <thread>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -123,6 +125,85 @@ std::string jsonDouble(double v) {
   std::string t(buf);
   if (t.find_first_of(".eEn") == std::string::npos) t += ".0";
   return t;
+}
+
+// Copies between pageable host memory and the pinned staging buffers on a few threads: one core moves about
+// 10 GB/s, the PCIe link several times that, so a single memcpy is what bounds the host path of small SPNs.
+class CopyCrew {
+ public:
+  static CopyCrew& instance() {
+    static CopyCrew* crew = new CopyCrew();  // never destroyed: its parked threads outlive static destruction
+    return *crew;
+  }
+  void copy(void* dst, const void* src, size_t bytes) {
+    const size_t parts = workers_.size() + 1;
+    if (bytes < (size_t(4) << 20) || parts == 1) {
+      std::memcpy(dst, src, bytes);
+      return;
+    }
+    std::lock_guard<std::mutex> serial(callMutex_);  // one copy at a time
+    const size_t share = (bytes / parts + 4095) & ~size_t(4095);
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      for (size_t w = 0; w < workers_.size(); ++w) {
+        const size_t lo = std::min(bytes, (w + 1) * share), hi = std::min(bytes, (w + 2) * share);
+        jobs_[w] = Job{static_cast<char*>(dst) + lo, static_cast<const char*>(src) + lo, hi - lo};
+      }
+      pending_ = workers_.size();
+      ++generation_;
+    }
+    wake_.notify_all();
+    std::memcpy(dst, src, std::min(bytes, share));
+    std::unique_lock<std::mutex> lock(mutex_);
+    done_.wait(lock, [&] { return pending_ == 0; });
+  }
+
+ private:
+  struct Job {
+    char* dst = nullptr;
+    const char* src = nullptr;
+    size_t bytes = 0;
+  };
+  CopyCrew() {
+    unsigned n = std::thread::hardware_concurrency();
+    n = n >= 8 ? 3 : (n >= 4 ? 1 : 0);  // the calling thread copies a share too
+    jobs_.resize(n);
+    for (unsigned w = 0; w < n; ++w) workers_.emplace_back([this, w] { run(w); });
+    for (auto& t : workers_) t.detach();
+  }
+  void run(unsigned w) {
+    uint64_t seen = 0;
+    for (;;) {
+      Job job;
+      {
+        std::unique_lock<std::mutex> lock(mutex_);
+        wake_.wait(lock, [&] { return generation_ != seen; });
+        seen = generation_;
+        job = jobs_[w];
+      }
+      if (job.bytes) std::memcpy(job.dst, job.src, job.bytes);
+      {
+        std::lock_guard<std::mutex> lock(mutex_);
+        if (--pending_ == 0) done_.notify_one();
+      }
+    }
+  }
+  std::vector<std::thread> workers_;
+  std::vector<Job> jobs_;
+  std::mutex mutex_, callMutex_;
+  std::condition_variable wake_, done_;
+  size_t pending_ = 0;
+  uint64_t generation_ = 0;
+};
+
+// True if `p` is host memory the GPU can copy from directly (hipHostMalloc / pinned), so that no staging copy is needed.
+bool isPinnedHost(const void* p) {
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+    (void)hipGetLastError();  // ordinary pageable memory is "invalid value" to the runtime
+    return false;
+  }
+  return attr.type == hipMemoryTypeHost;
 }
 
 std::string makeKernelFilePath() {
@@ -636,10 +717,14 @@ void Kernel::execute(size_t n, const void* in, void* out) {
   size_t chunk = std::max<size_t>(4096, (size_t(32) << 20) / std::max<size_t>(1, rowBytes));
   chunk = std::min(chunk, n);
   ensureStaging(chunk);
+  // Buffers the caller has pinned are copied from / to directly; pageable ones go through the pinned staging
+  // buffers, filled by a few threads.
+  const bool pinnedIn = isPinnedHost(in), pinnedOut = isPinnedHost(out);
+  CopyCrew& crew = CopyCrew::instance();
   auto drain = [&](Stage& s) {
     if (!s.pendingRows) return;
     hipCheck(hipStreamSynchronize(s.stream), "hipStreamSynchronize");
-    std::memcpy(static_cast<char*>(out) + s.pendingOffset * bytesPerResult_, s.hOut, s.pendingRows * bytesPerResult_);
+    if (!pinnedOut) std::memcpy(static_cast<char*>(out) + s.pendingOffset * bytesPerResult_, s.hOut, s.pendingRows * bytesPerResult_);
     s.pendingRows = 0;
   };
   size_t done = 0;
@@ -649,14 +734,19 @@ void Kernel::execute(size_t n, const void* in, void* out) {
       Stage& s = stage_[turn & 1];
       drain(s);
       const size_t rows = std::min(chunk, n - done);
-      std::memcpy(s.hIn, static_cast<const char*>(in) + done * rowBytes, rows * rowBytes);
-      hipCheck(hipMemcpyAsync(s.dIn, s.hIn, rows * rowBytes, hipMemcpyHostToDevice, s.stream), "input copy");
+      const char* src = static_cast<const char*>(in) + done * rowBytes;
+      if (!pinnedIn) {
+        crew.copy(s.hIn, src, rows * rowBytes);
+        src = static_cast<const char*>(s.hIn);
+      }
+      hipCheck(hipMemcpyAsync(s.dIn, src, rows * rowBytes, hipMemcpyHostToDevice, s.stream), "input copy");
       // Kernels of successive chunks run one after the other (they share the spill buffer);
       // only the copies overlap them.
       if (turn) hipCheck(hipStreamWaitEvent(s.stream, kernelDone_, 0), "hipStreamWaitEvent");
       launch(rows, s.dIn, s.dOut, s.stream);
       hipCheck(hipEventRecord(kernelDone_, s.stream), "hipEventRecord");
-      hipCheck(hipMemcpyAsync(s.hOut, s.dOut, rows * bytesPerResult_, hipMemcpyDeviceToHost, s.stream), "output copy");
+      void* dst = pinnedOut ? static_cast<void*>(static_cast<char*>(out) + done * bytesPerResult_) : s.hOut;
+      hipCheck(hipMemcpyAsync(dst, s.dOut, rows * bytesPerResult_, hipMemcpyDeviceToHost, s.stream), "output copy");
       s.pendingRows = rows;
       s.pendingOffset = done;
       done += rows;
