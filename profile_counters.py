@@ -5,7 +5,7 @@ For every benchmark configuration it runs bench.py under rocprofv3 (kernel trace
 FETCH_SIZE and WRITE_SIZE, then two sets of SQ counters), each in a pass of its own, and writes
 
   profiles/<kernel>_<config>.txt   the figures, with the command of every pass
-  profiles/copy_1gib_counters.txt  what the traffic counters read for a plain 1 GiB device copy (their calibration)
+  profiles/copy_kernel_counters.txt  what the traffic counters read for a plain 4 GiB device copy (their calibration)
   profiles/traffic.json            HBM bytes per launch per configuration, with bench.py's key of the kernel measured
 
 usage: python3 profile_counters.py [config ...]       (default: all six; raw profiler output goes to a temporary directory)
@@ -66,13 +66,14 @@ def main():
     # ---- calibration: what the traffic counters read for a copy of known size ----
     units, copy_lines = {}, []
     for counter in ("FETCH_SIZE", "WRITE_SIZE"):
-        con, _, shown = rocprof(work, "copy_" + counter, ["--pmc", counter], ["--copy-gib", "1", "--steps", "5"])
+        con, _, shown = rocprof(work, "copy_" + counter, ["--pmc", counter], ["--copy-gib", "4", "--steps", "5"])
         value = max(r[1] for r in counters(con, "%"))
-        units[counter] = 1048576.0 / value          # KiB per counter unit
+        units[counter] = 4 * 1048576.0 / value      # KiB per counter unit
         copy_lines += ["$ " + shown, "%-46s %-12s per-dispatch=%.1f" % ("copy kernel", counter, value)]
-    with open(os.path.join(prof, "copy_1gib_counters.txt"), "w") as f:
-        f.write("Plain device-to-device copy of 1 GiB (torch Tensor.copy_), the reference point for the FETCH_SIZE and WRITE_SIZE\n"
-                "counters of rocprofv3 on MI355X: the copy reads 1 GiB and writes 1 GiB (1048576 KiB each).\n"
+    with open(os.path.join(prof, "copy_kernel_counters.txt"), "w") as f:
+        f.write("Plain device-to-device copy of 4 GiB (torch Tensor.copy_), the reference point for the FETCH_SIZE and WRITE_SIZE\n"
+                "counters of rocprofv3 on MI355X: the copy reads 4 GiB and writes 4 GiB (4194304 KiB each; far more than the 256 MiB\n"
+                "of last-level cache could hold back from HBM).\n"
                 "Made by: python3 profile_counters.py\n\n" + "\n".join(copy_lines) +
                 "\n\nOne FETCH_SIZE unit is %.3f KiB, one WRITE_SIZE unit %.3f KiB.\n" % (units["FETCH_SIZE"], units["WRITE_SIZE"]))
     try:
@@ -104,7 +105,7 @@ def main():
         text += ["", "bench.py, same run as the kernel trace: %.4g samples/s, launch %.4f ms (HIP events); rocprofv3 average %.4f ms."
                  % (line["value"], roof["launch_ms"], avg_ns / 1e6),
                  "roofline bound %s, achieved %s of %s %s = %s." % (roof["bound"], roof["achieved"], roof["peak"], roof["unit"], roof["frac"]),
-                 "Counter calibration (profiles/copy_1gib_counters.txt): FETCH_SIZE x %.3f, WRITE_SIZE x %.3f give KiB of HBM traffic."
+                 "Counter calibration (profiles/copy_kernel_counters.txt): FETCH_SIZE x %.3f, WRITE_SIZE x %.3f give KiB of HBM traffic."
                  % (units["FETCH_SIZE"], units["WRITE_SIZE"]),
                  "HBM traffic per launch: %.3f GiB; algorithmic bytes (inputs + results) %.3f GiB; ratio %.3f."
                  % (hbm_bytes / 2 ** 30, algorithmic / 2 ** 30, hbm_bytes / algorithmic), "",

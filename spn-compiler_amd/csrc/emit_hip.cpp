@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <map>
 #include <sstream>
 #include <stdexcept>
 #include <unordered_map>
@@ -49,6 +50,29 @@ struct Emitter {
   std::vector<bool> emitted;
   std::unordered_map<uint32_t, double> foldedWeight;
   bool vectorRows = true;
+  // Packed rows: the row reaches the kernel body as F/4 registers holding four features each, one byte per feature
+  // (the value itself, saturated at 255). Table leaves that only their product reads are evaluated per group of sibling
+  // products (the products under one sum that cover the same features), feature by feature: leaves over two or three
+  // categories as polynomials in the feature's value (multiply-adds, no memory), the others from joint tables over pairs
+  // of features in LDS, one index per pair for all siblings, whose entries lie side by side.
+  bool packedRows = false;
+  bool clampPacked = true;             // clamp the packed bytes to their tables' lengths before they index LDS
+  std::vector<bool> featOneHot;        // per feature: its leaves are evaluated without memory accesses
+  struct FusedUnit {
+    uint32_t fa = 0, fb = UINT32_MAX;  // one feature, or a pair with a joint table
+    uint32_t rowsA = 1, rowsB = 1;
+    uint32_t base = 0, stride = 1;     // pool offset of the unit's table; entries per index (the siblings, padded to an even count)
+  };
+  struct FusedGroup {
+    std::vector<uint32_t> products;                    // the siblings
+    std::vector<std::map<uint32_t, uint32_t>> leafOf;  // per sibling: feature -> leaf node
+    std::vector<uint32_t> hot;                         // features evaluated from one-hot factors
+    std::vector<FusedUnit> units;                      // features read from LDS
+    bool emitted = false;
+  };
+  std::vector<FusedGroup> fusedGroups;
+  std::vector<int> fusedGroupOf;       // per node: group of a product whose table leaves are evaluated this way, or -1
+  std::vector<bool> fusedLeaf;         // per node: table leaf evaluated inside its product's group
 
   Emitter(const Graph& graph, const CompileOptions& opts) : g(graph), o(opts) {
     logSpace = o.useLogSpace;
@@ -119,6 +143,10 @@ struct Emitter {
     // The index is clamped once per feature.
     tableOffset.assign(g.nodes.size(), 0);
     partner.assign(g.nodes.size(), UINT32_MAX);
+    fusedGroupOf.assign(g.nodes.size(), -1);
+    fusedLeaf.assign(g.nodes.size(), false);
+    featOneHot.assign(g.numFeatures, false);
+    if (packedRows) planFusedGroups();
     auto isTable = [&](uint32_t c) { return g.nodes[c].kind == NodeKind::Categorical || g.nodes[c].kind == NodeKind::Histogram; };
     auto rowLen = [&](uint32_t feature) { return size_t(featTableLen[feature]) + (g.supportMarginal ? 2 : 1); };
     // Joint tables: two table leaves read only by the same product are replaced by one table over
@@ -136,7 +164,7 @@ struct Emitter {
       uint32_t a, b;
     };
     std::vector<Candidate> candidates;
-    for (uint32_t i = 0; i < g.nodes.size() && o.jointTables; ++i) {
+    for (uint32_t i = 0; i < g.nodes.size() && o.jointTables && !packedRows; ++i) {
       if (g.nodes[i].kind != NodeKind::Product) continue;
       std::vector<uint32_t> leaves;
       for (uint32_t c : g.nodes[i].children)
@@ -158,16 +186,359 @@ struct Emitter {
     }
     // Units (single tables and joint tables) by index, in node order.
     for (uint32_t i = 0; i < g.nodes.size(); ++i) {
-      if (!isTable(i)) continue;
+      if (!isTable(i) || fusedLeaf[i]) continue;
       if (partner[i] != UINT32_MAX && partner[i] < i) continue;  // second leaf of a pair: lives in the joint table
       const uint64_t fb = partner[i] == UINT32_MAX ? 0 : uint64_t(g.nodes[partner[i]].feature) + 1;
-      const uint64_t key = o.groupedTables ? (uint64_t(g.nodes[i].feature) << 32) | fb : uint64_t(i);  // ungrouped: every table on its own
+      const uint64_t key = o.groupedTables && !packedRows ? (uint64_t(g.nodes[i].feature) << 32) | fb : uint64_t(i);  // ungrouped: every table on its own
       if (!unitsByKey.count(key)) keyOrder.push_back(key);
       unitsByKey[key].push_back(i);
     }
     useRank.assign(g.nodes.size(), 0);
-    if (o.groupedTables && !unitsByKey.empty()) recordUseOrder();
+    if (o.groupedTables && !packedRows && !unitsByKey.empty()) recordUseOrder();
     buildPool();
+    if (packedRows) appendFusedTables();
+  }
+
+  // ---- packed rows: groups of sibling products ----
+  bool isTableLeaf(uint32_t c) const { return g.nodes[c].kind == NodeKind::Categorical || g.nodes[c].kind == NodeKind::Histogram; }
+  // Entries per feature in the tables of the groups: no "impossible" entry. An input outside a feature's range is found
+  // by a test of its own on the packed registers and makes the kernel return log 0; its clamped index reads one entry
+  // past its table, inside the pool (which ends in padding), and whatever comes of that is dropped.
+  uint32_t rowsOf(uint32_t feature) const { return featTableLen[feature]; }
+  // Entries per index of a group's tables: the siblings' values side by side, padded to an even count so that two
+  // of them are one aligned 8-byte (float) or 16-byte (double) LDS read.
+  // The count of such reads per index is made odd: with an even count, entries 32 / count apart (or a fraction of
+  // that) start in the same LDS bank, and lanes that read different entries of one table wait for each other (measured
+  // on a graph with groups of four and eight siblings: 44 % of the LDS cycles were bank conflicts).
+  static size_t fusedStride(size_t siblings) {
+    if (siblings == 1) return 1;
+    const size_t reads = (siblings + 1) / 2;
+    return 2 * (reads | 1);
+  }
+
+  void planFusedGroups() {
+    std::vector<uint32_t> parent(g.nodes.size(), UINT32_MAX);
+    for (uint32_t i = 0; i < g.nodes.size(); ++i)
+      for (uint32_t c : g.nodes[i].children) parent[c] = i;
+    // One-hot features: few categories, and every leaf on the feature has a finite value for each of them.
+    for (uint32_t f = 0; f < g.numFeatures; ++f) featOneHot[f] = featTableLen[f] != 0 && featTableLen[f] <= uint32_t(o.oneHotMaxDomain);
+    for (const auto& n : g.nodes) {
+      if (n.kind != NodeKind::Categorical && n.kind != NodeKind::Histogram) continue;
+      bool finite = n.table.size() == featTableLen[n.feature];
+      for (double p : n.table) finite = finite && p > 0;
+      if (!finite) featOneHot[n.feature] = false;
+    }
+    std::map<std::pair<uint32_t, std::vector<uint32_t>>, size_t> byKey;
+    for (uint32_t i = 0; i < g.nodes.size(); ++i) {
+      if (g.nodes[i].kind != NodeKind::Product) continue;
+      std::map<uint32_t, uint32_t> own;  // feature -> leaf
+      bool distinct = true;
+      for (uint32_t c : g.nodes[i].children)
+        if (isTableLeaf(c) && g.nodes[c].uses == 1) distinct = own.emplace(g.nodes[c].feature, c).second && distinct;
+      if (own.empty() || !distinct) continue;
+      std::vector<uint32_t> features;
+      for (const auto& kv : own) features.push_back(kv.first);
+      const bool underSum = g.nodes[i].uses == 1 && parent[i] != UINT32_MAX && g.nodes[parent[i]].kind == NodeKind::Sum;
+      const auto key = std::make_pair(underSum ? parent[i] : uint32_t(g.nodes.size()) + i, features);
+      auto it = byKey.find(key);
+      if (it == byKey.end()) {
+        it = byKey.emplace(key, fusedGroups.size()).first;
+        FusedGroup G;
+        std::vector<uint32_t> lds;
+        for (uint32_t f : features) (featOneHot[f] ? G.hot : lds).push_back(f);
+        std::stable_sort(lds.begin(), lds.end(), [&](uint32_t x, uint32_t y) { return rowsOf(x) < rowsOf(y); });
+        for (size_t k = 0; k < lds.size();) {
+          FusedUnit u;
+          u.fa = lds[k];
+          u.rowsA = rowsOf(lds[k]);
+          if (o.jointTables && k + 1 < lds.size() && size_t(u.rowsA) * rowsOf(lds[k + 1]) <= size_t(o.jointMaxEntries)) {
+            u.fb = lds[k + 1];
+            u.rowsB = rowsOf(lds[k + 1]);
+            k += 2;
+          } else {
+            k += 1;
+          }
+          G.units.push_back(u);
+        }
+        fusedGroups.push_back(std::move(G));
+      }
+      FusedGroup& G = fusedGroups[it->second];
+      G.products.push_back(i);
+      G.leafOf.push_back(own);
+      fusedGroupOf[i] = int(it->second);
+      for (const auto& kv : own) fusedLeaf[kv.second] = true;
+    }
+    // The joint tables must fit beside everything else in LDS: the largest pairs are split again until they do.
+    size_t other = 0;
+    for (uint32_t i = 0; i < g.nodes.size(); ++i)
+      if (isTableLeaf(i) && !fusedLeaf[i]) other += rowsOf(g.nodes[i].feature);
+    auto total = [&] {
+      size_t t = other;
+      for (const auto& G : fusedGroups)
+        for (const auto& u : G.units) t += fusedStride(G.products.size()) * size_t(u.rowsA) * u.rowsB;
+      return t;
+    };
+    const size_t budget = size_t(o.tableBudgetGiven ? o.tableBudgetKiB : 80) * 1024 / (f64 ? 8 : 4);
+    while (total() > budget) {
+      FusedGroup* bestG = nullptr;
+      size_t bestU = 0, bestGain = 0;
+      for (auto& G : fusedGroups)
+        for (size_t k = 0; k < G.units.size(); ++k) {
+          const FusedUnit& u = G.units[k];
+          if (u.fb == UINT32_MAX) continue;
+          const size_t gain = fusedStride(G.products.size()) * (size_t(u.rowsA) * u.rowsB - u.rowsA - u.rowsB);
+          if (gain > bestGain) bestGain = gain, bestG = &G, bestU = k;
+        }
+      if (!bestG) break;
+      FusedUnit second;
+      second.fa = bestG->units[bestU].fb;
+      second.rowsA = bestG->units[bestU].rowsB;
+      bestG->units[bestU].fb = UINT32_MAX;
+      bestG->units[bestU].rowsB = 1;
+      bestG->units.insert(bestG->units.begin() + bestU + 1, second);
+    }
+  }
+
+  // Per unit one table whose entry `index` holds the values of all siblings side by side: one address serves them all
+  // and two neighbours come with one read.
+  void appendFusedTables() {
+    auto padded = [&](uint32_t leaf) {
+      const auto& n = g.nodes[leaf];
+      std::vector<double> t;
+      for (uint32_t j = 0; j < rowsOf(n.feature); ++j) t.push_back(logConst(j < n.table.size() ? n.table[j] : 0.0));
+      return t;
+    };
+    // The bytes of a packed row are saturated at the longest table's length when the row is packed, so an index made of
+    // unclamped bytes reaches at most `reach` entries past the start of its table. With that much padding behind the
+    // pool no byte needs a clamp of its own: an input outside its feature's range makes the kernel return log 0
+    // whatever the tables gave. When the padding would be large the bytes are clamped instead, and a clamped
+    // out-of-range index reads at most one row of the first feature past its table.
+    size_t largestRow = 0, reach = 0;
+    for (auto& G : fusedGroups)
+      for (auto& u : G.units) {
+        const size_t k = G.products.size();
+        u.stride = uint32_t(fusedStride(k));
+        if (tablePool.size() % 2) tablePool.push_back(0.0);
+        u.base = uint32_t(tablePool.size());
+        const size_t entries = size_t(u.rowsA) * u.rowsB;
+        tablePool.resize(tablePool.size() + entries * u.stride, 0.0);
+        for (size_t j = 0; j < k; ++j) {
+          const std::vector<double> a = padded(G.leafOf[j].at(u.fa));
+          const std::vector<double> b = u.fb == UINT32_MAX ? std::vector<double>{0.0} : padded(G.leafOf[j].at(u.fb));
+          for (size_t x = 0; x < a.size(); ++x)
+            for (size_t y = 0; y < b.size(); ++y) tablePool[u.base + (x * b.size() + y) * u.stride + j] = a[x] + b[y];
+        }
+        largestRow = std::max(largestRow, size_t(u.rowsB + 1) * u.stride);
+        reach = std::max(reach, size_t(packedSaturation()) * size_t(u.rowsB + 1) * u.stride);
+      }
+    reach = std::max(reach, size_t(packedSaturation()) + 1);  // leaves outside the groups index their tables with the byte itself
+    clampPacked = reach * (f64 ? 8 : 4) > 8192;
+    if (!fusedGroups.empty()) tablePool.resize(tablePool.size() + (clampPacked ? largestRow : reach) + 2, 0.0);
+  }
+  // What a value is saturated at when a row is packed: the longest table's length, which is out of every feature's range.
+  uint32_t packedSaturation() const {
+    uint32_t longest = 1;
+    for (uint32_t f = 0; f < g.numFeatures; ++f) longest = std::max(longest, featTableLen[f]);
+    return longest;
+  }
+
+  unsigned extractions2 = 0;
+  static std::string byteSel(uint32_t f) { return "BYTE_" + std::to_string(f % 4); }
+  // Byte f of the packed row times a constant, as one instruction (the operand's byte select does the extraction).
+  // Written as a volatile statement: these stay in program order, so an index exists only from where the generator
+  // put it. Left to the compiler, the extractions are merged or moved to the top of the kernel, and hundreds of
+  // indices stay in registers (measured: 256 registers and 470 spilled ones against 140).
+  std::string packedByteTimes(uint32_t f, size_t factor) {
+    const std::string name = "e" + std::to_string(extractions2++);
+    body << "  unsigned " << name << ";\n  asm volatile(\"v_mul_u32_u24_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:" << byteSel(f)
+         << " src1_sel:DWORD\" : \"=v\"(" << name << ") : \"v\"(PK" << f / 4 << "), \"s\"(" << factor << "u));\n";
+    return name;
+  }
+  std::string packedByte(uint32_t f) {
+    const std::string name = "e" + std::to_string(extractions2++);
+    body << "  unsigned " << name << ";\n  asm volatile(\"v_bfe_u32 %0, %1, " << 8 * (f % 4) << ", 8\" : \"=v\"(" << name << ") : \"v\"(PK" << f / 4 << "));\n";
+    return name;
+  }
+
+  // What the kernel body starts with when rows are packed: the test for inputs outside their feature's range (in a
+  // complete and decomposable graph such an input makes the result log 0, which the kernel returns at the end), the
+  // clamp of the bytes where it is needed, and the values of the features whose leaves are polynomials.
+  void emitPackedPrologue() {
+    // Range test on the four bytes of a register at once: for a byte x and its length L <= 128,
+    // ((x & 0x7f) + (0x80 - L)) | x has its top bit set exactly when x >= L (no carry leaves a byte).
+    body << "  unsigned outsideBits = 0u;\n";
+    for (uint32_t c = 0; c * 4 < g.numFeatures; ++c) {
+      unsigned add = 0, keep = 0;
+      for (uint32_t j = 0; j < 4 && c * 4 + j < g.numFeatures; ++j) {
+        const uint32_t f = c * 4 + j;
+        if (!featTableLen[f]) continue;
+        keep |= 0xffu << (8 * j);
+        add |= (0x80u - featTableLen[f]) << (8 * j);
+      }
+      if (!keep) continue;
+      const std::string x = "R[" + std::to_string(c) + "]";
+      body << "  outsideBits |= (((" << x << " & 0x7f7f7f7fu) + " << add << "u) | " << x << ")" << (keep != 0xffffffffu ? " & " + std::to_string(keep) + "u" : std::string())
+           << ";\n";
+    }
+    body << "  const bool outside = (outsideBits & 0x80808080u) != 0u;\n";
+    // Clamp: one byte-wise minimum per feature, in place (the other bytes of the register are preserved). Written as
+    // instructions: from the equivalent C expression the compiler makes about six instructions per feature. Left out
+    // when even an index made of arbitrary bytes stays inside the kernel's LDS: what such a read returns is dropped.
+    for (uint32_t c = 0; c * 4 < g.numFeatures; ++c) {
+      std::string clamp, operands;
+      unsigned operand = 1;
+      for (uint32_t j = 0; j < 4 && c * 4 + j < g.numFeatures; ++j) {
+        const uint32_t f = c * 4 + j;
+        if (!featTableLen[f]) continue;
+        clamp += std::string(clamp.empty() ? "" : "\\n\\t") + "v_min_u32_sdwa %0, %0, %" + std::to_string(operand++) + " dst_sel:BYTE_" + std::to_string(j) +
+                 " dst_unused:UNUSED_PRESERVE src0_sel:BYTE_" + std::to_string(j) + " src1_sel:DWORD\\n\\ts_nop 0";  // a partial write, then a wait state
+        operands += std::string(operands.empty() ? "" : ", ") + "\"s\"(" + std::to_string(featTableLen[f]) + "u)";
+      }
+      if (clamp.empty()) continue;
+      body << "  unsigned PK" << c << " = R[" << c << "];\n";
+      if (clampPacked) body << "  asm(\"" << clamp << "\" : \"+v\"(PK" << c << ") : " << operands << ");\n";
+    }
+    for (uint32_t f = 0; f < g.numFeatures && o.hoistFeatureValues; ++f)
+      if (featOneHot[f]) emitFeatureValues(f, "");
+  }
+
+  // x (and x squared, or the 0/1 factors [x == c]) of a feature whose leaves are evaluated without memory accesses.
+  void emitFeatureValues(uint32_t f, const std::string& suffix) {
+    const char* one = f64 ? "1.0" : "1.0f";
+    const char* zero = f64 ? "0.0" : "0.0f";
+    const uint32_t d = featTableLen[f];
+    const std::string v = "h" + std::to_string(f) + "_1" + suffix;
+    if (!f64 && !suffix.empty())  // inside a group: as a volatile statement, or the compiler computes all of them at the top of the kernel again
+      body << "  real_t " << v << ";\n  asm volatile(\"v_cvt_f32_ubyte" << f % 4 << " %0, %1\" : \"=v\"(" << v << ") : \"v\"(PK" << f / 4 << "));\n";
+    else
+      body << "  const real_t " << v << " = (real_t)((PK" << f / 4 << " >> " << 8 * (f % 4) << ") & 255u);\n";  // one instruction: byte to float
+    if (d == 3) body << "  const real_t h" << f << "_2" << suffix << " = " << v << " * " << v << ";\n";
+    for (uint32_t c = 2; d > 3 && c < d; ++c)
+      body << "  const real_t h" << f << "_" << c << suffix << " = " << v << " == " << lit(double(c)) << " ? " << one << " : " << zero << ";\n";
+  }
+
+  // The table leaves of a group of sibling products, into one accumulator per sibling (named pt<product>).
+  bool midpointHook = false;      // the body calls spn_mid() once, about half-way through its work (the row prefetch turns round there)
+  bool midpointEmitted = false;
+  size_t fusedWorkDone = 0;
+  static size_t workOf(const FusedGroup& G) { return G.products.size() * (G.units.size() + 2 * G.hot.size()); }
+
+  void emitFusedGroup(FusedGroup& G) {
+    G.emitted = true;
+    const size_t k = G.products.size();
+    if (midpointHook && !midpointEmitted) {
+      size_t total = 0;
+      for (const auto& other : fusedGroups) total += workOf(other);
+      if (2 * fusedWorkDone >= total) {
+        body << "  spn_mid();\n";
+        midpointEmitted = true;
+      }
+    }
+    fusedWorkDone += workOf(G);
+    const size_t realBytes = f64 ? 8 : 4;
+    const char* fma = f64 ? "__builtin_fma(" : "__builtin_fmaf(";
+    // Few siblings mean few independent chains of dependent adds, and with two wavefronts per SIMD nothing else hides
+    // the latency of a vector instruction: each sibling's sum is then split over several partial accumulators.
+    const size_t parts = k >= 4 ? 1 : (k == 3 ? 2 : (k == 2 ? 2 : 4));
+    std::vector<std::vector<std::string>> acc(k);
+    std::vector<std::string> allAcc;
+    std::vector<size_t> turn(k, 0);
+    for (size_t j = 0; j < k; ++j) {
+      double base = 0;
+      for (uint32_t f : G.hot) base += logConst(g.nodes[G.leafOf[j].at(f)].table[0]);
+      for (size_t q = 0; q < parts; ++q) {
+        acc[j].push_back("pt" + std::to_string(G.products[j]) + (q ? "_" + std::to_string(q) : std::string()));
+        body << "  real_t " << acc[j].back() << " = " << lit(q ? 0.0 : base) << ";\n";
+        allAcc.push_back(acc[j].back());
+      }
+      for (const auto& kv : G.leafOf[j]) emitted[kv.second] = true;
+    }
+    auto next = [&](size_t j) -> const std::string& { return acc[j][turn[j]++ % parts]; };
+    // Work that needs no memory. A leaf over two or three categories is the polynomial through its values at x = 0, 1
+    // (and 2): value(0) is part of the accumulator's start, the rest is one multiply-add per power of x. A leaf over
+    // more categories (on request) is value(0) + (value(1) - value(0)) x plus one correction per category c >= 2,
+    // multiplied with the 0/1 factor [x == c].
+    std::vector<std::string> hotWork;
+    const std::string suffix = o.hoistFeatureValues ? std::string() : "_g" + std::to_string(G.products[0]);
+    for (uint32_t f : G.hot) {
+      const uint32_t d = featTableLen[f];
+      if (!o.hoistFeatureValues) emitFeatureValues(f, suffix);
+      for (size_t j = 0; j < k; ++j) {
+        const auto& t = g.nodes[G.leafOf[j].at(f)].table;
+        const double v0 = logConst(t[0]), v1 = logConst(t[1]);
+        std::vector<double> factor(d, 0.0);  // coefficient of h<f>_<c>
+        if (d == 2) {
+          factor[1] = v1 - v0;
+        } else if (d == 3) {
+          const double v2 = logConst(t[2]);
+          factor[2] = (v2 - 2 * v1 + v0) / 2;
+          factor[1] = v1 - v0 - factor[2];
+        } else {
+          // x = h_1 is the value itself: value(x) = v0 + (v1 - v0) * x + sum over c >= 2 of (v_c - v0 - c (v1 - v0)) [x == c]
+          factor[1] = v1 - v0;
+          for (uint32_t c = 2; c < d; ++c) factor[c] = logConst(t[c]) - v0 - double(c) * factor[1];
+        }
+        for (uint32_t c = 1; c < d; ++c) {
+          const std::string& a = next(j);
+          hotWork.push_back("  " + a + " = " + fma + "h" + std::to_string(f) + "_" + std::to_string(c) + suffix + ", " + lit(factor[c]) + ", " + a + ");\n");
+        }
+      }
+    }
+    // LDS reads in batches: the indices and reads of a batch are issued, then the values of the batch before are
+    // added (and a share of the other work done) while they travel.
+    const int fusedBatch = o.fusedBatch >= 0 ? o.fusedBatch : (midpointHook ? 2 : 4);
+    const size_t batch = size_t(std::max(1, fusedBatch)), batches = (G.units.size() + batch - 1) / batch;
+    const bool barriers = fusedBatch > 0;
+    const size_t hotShare = batches ? (hotWork.size() + batches - 1) / batches : hotWork.size();
+    size_t hotDone = 0;
+    std::vector<std::string> pendingAdds;
+    // Empty volatile statements that take the accumulators in and out: volatile statements keep their order (the
+    // index computations are volatile too), so the adds between two of these pins stay between this batch's reads and
+    // the next batch's indices. A scheduling barrier alone does not bind the compiler before instruction selection.
+    auto pin = [&] {
+      for (const std::string& a : allAcc) body << "  asm volatile(\"\" : \"+v\"(" << a << "));\n";
+      body << "  __builtin_amdgcn_sched_barrier(0);\n";
+    };
+    for (size_t b0 = 0; b0 < G.units.size(); b0 += batch) {
+      std::vector<std::string> adds;
+      for (size_t q = b0; q < std::min(G.units.size(), b0 + batch); ++q) {
+        const FusedUnit& u = G.units[q];
+        // Byte offset of the unit's entry: (a * rowsB + b) * stride * sizeof(real_t), one multiply per feature.
+        std::string idx = packedByteTimes(u.fa, size_t(u.rowsB) * u.stride * realBytes);
+        if (u.fb != UINT32_MAX) {
+          const std::string second = packedByteTimes(u.fb, u.stride * realBytes);
+          const std::string joint = "j" + std::to_string(extractions2++);
+          body << "  const unsigned " << joint << " = " << idx << " + " << second << ";\n";
+          idx = joint;
+        }
+        for (size_t j = 0; j < k; j += 2) {
+          const std::string r = "r" + std::to_string(extractions2++);
+          const std::string address = "reinterpret_cast<const char*>(tab + " + std::to_string(u.base + j) + "u) + " + idx;
+          if (u.stride == 1) {
+            body << "  const real_t " << r << " = *reinterpret_cast<const real_t*>(" << address << ");\n";
+            adds.push_back("  " + next(j) + " += " + r + ";\n");
+          } else {
+            body << "  const spn_r2 " << r << " = *reinterpret_cast<const spn_r2*>(" << address << ");\n";
+            adds.push_back("  " + next(j) + " += " + r + "[0];\n");
+            if (j + 1 < k) adds.push_back("  " + next(j + 1) + " += " + r + "[1];\n");
+          }
+        }
+      }
+      if (!barriers) {  // plain order: every unit's values are added right after its reads
+        for (const std::string& a : adds) body << a;
+        for (size_t q = 0; q < hotShare && hotDone < hotWork.size(); ++q) body << hotWork[hotDone++];
+        continue;
+      }
+      pin();
+      for (const std::string& a : pendingAdds) body << a;
+      for (size_t q = 0; q < hotShare && hotDone < hotWork.size(); ++q) body << hotWork[hotDone++];
+      pin();
+      pendingAdds = std::move(adds);
+    }
+    for (const std::string& a : pendingAdds) body << a;
+    while (hotDone < hotWork.size()) body << hotWork[hotDone++];
+    for (size_t j = 0; j < k; ++j)
+      for (size_t q = 1; q < parts; ++q) body << "  " << acc[j][0] << " += " << acc[j][q] << ";\n";
   }
 
   std::vector<double> unitValues(uint32_t i) const {
@@ -371,6 +742,11 @@ struct Emitter {
     {
       if (featPrepared[f]) return;
       featPrepared[f] = true;
+      if (packedRows) {  // a leaf outside the groups: the clamped index itself
+        const std::string x = packedByte(f);
+        body << "  const unsigned t" << f << " = " << x << ";\n";
+        return;
+      }
       std::string x = "x[" + std::to_string(f) + "]";
       if (!vectorRows) {
         body << "  const feat_t x" << f << " = SPN_LOAD(row + " << f << ");\n";
@@ -433,6 +809,7 @@ struct Emitter {
   std::vector<std::string> productOperands(const std::vector<uint32_t>& kids) {
     std::vector<std::string> ops;
     for (uint32_t c : kids) {
+      if (fusedLeaf[c]) continue;  // part of pt<product>, which the caller adds
       const bool table = g.nodes[c].kind == NodeKind::Categorical || g.nodes[c].kind == NodeKind::Histogram;
       if (!table || partner[c] == UINT32_MAX) {
         emitNode(c);
@@ -534,7 +911,9 @@ struct Emitter {
           break;
         }
         const char* op = logSpace ? " + " : " * ";
-        const std::vector<std::string> ops = productOperands(n.children);
+        if (fusedGroupOf[i] >= 0 && !fusedGroups[size_t(fusedGroupOf[i])].emitted) emitFusedGroup(fusedGroups[size_t(fusedGroupOf[i])]);
+        std::vector<std::string> ops = productOperands(n.children);
+        if (fusedGroupOf[i] >= 0) ops.push_back("pt" + std::to_string(i));
         std::string e = tree(
             0, ops.size(), [&](size_t k) { return ops[k]; },
             [&](const std::string& a, const std::string& b) { return "(" + a + op + b + ")"; });
@@ -638,6 +1017,21 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   // Short rows are fetched with the widest vector loads their size allows, all samples of a
   // lane up front; wide rows are read feature by feature next to the first use.
   e.vectorRows = g.numFeatures * g.ftype.bytes <= 512;
+  {
+    // Packed rows: wide rows of 32-bit integers that only feed table leaves with short tables, in a complete and
+    // decomposable graph (an input outside a one-hot feature's range is reported through a flag, not through a table).
+    bool eligible = e.logSpace && e.vectorRows && !g.ftype.isFloat && g.ftype.bytes == 4 && g.numFeatures % 4 == 0 &&
+                    g.numFeatures * 4 >= 128 && g.completeDecomposable && !g.supportMarginal && o.samplesPerLane <= 1;
+    bool anyTable = false;
+    for (const auto& n : g.nodes) {
+      if (n.kind == NodeKind::Gaussian) eligible = false;
+      if (n.kind == NodeKind::Categorical || n.kind == NodeKind::Histogram) {
+        anyTable = true;
+        if (n.table.size() > 128) eligible = false;  // the range test on packed bytes handles lengths up to 128
+      }
+    }
+    e.packedRows = eligible && anyTable && o.packedRows != 0 && o.waveTranspose != 0;  // packed rows come out of the per-wavefront transposed load
+  }
   e.prepare();
   JitSource js;
   js.entry = "spn_kernel";
@@ -658,6 +1052,12 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   // Rows held in registers: the clamped table indices are derived right away, so that a raw feature
   // value and its index are never live together for long.
   auto emitBody = [&] {
+    if (e.packedRows) {
+      e.emitPackedPrologue();
+      e.emitNode(g.root());
+      if (e.midpointHook && !e.midpointEmitted) e.body << "  spn_mid();\n";
+      return;
+    }
     if (e.vectorRows && o.eagerIndices)
       for (uint32_t f = 0; f < F; ++f)
         if (e.featUsed[f] && e.featTableLen[f]) e.emitFeaturePrep(f);
@@ -673,7 +1073,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   const size_t work = g.nodes.size() + g.stats.sumTerms;
   unsigned U = unsigned(o.samplesPerLane);
   if (U == 0) U = (work <= 4000 && !g.supportMarginal && size_t(js.tableEntries) * realBytes <= 16 * 1024) ? 2 : 1;
-  if (!e.vectorRows) U = 1;
+  if (!e.vectorRows || e.packedRows) U = 1;
   js.samplesPerLane = U;
   // Kernels that sit on the HBM bound and stage their input tile through LDS run 2-3 % faster with
   // 512-thread blocks (measured on the six-feature product: 0.82 against 0.80 of the HBM peak).
@@ -697,7 +1097,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     bool eligible = e.vectorRows && !g.ftype.isFloat && eb == 4 && F % 4 == 0 && U == 1 && rowBytes >= 128;
     for (uint32_t f = 0; f < F && eligible; ++f)
       if (e.featGauss[f] || e.featTableLen[f] > 255) eligible = false;
-    if (eligible && o.waveTranspose == 1) {  // measured on the 100-feature discrete graphs: no gain yet beside unpacked indices (0.79 against 0.78 ms), so only on request
+    if (eligible && (o.waveTranspose == 1 || (e.packedRows && o.waveTranspose != 0))) {  // beside unpacked indices it gains nothing (0.79 against 0.78 ms on the 100-feature discrete graph): only with packed rows, or on request
       waveStride = (F / 4) | 1u;
       const size_t tables = js.tablesInLds ? size_t(js.tableEntries) * realBytes : 0;
       unsigned block = o.blockSize ? unsigned(o.blockSize) : 512u;
@@ -709,6 +1109,12 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     }
   }
   js.waveTransposedInput = waveTile;
+  js.packedRows = e.packedRows && waveTile;
+  if (e.packedRows && !waveTile) {  // the row buffers do not fit beside the tables: the same kernel with unpacked rows
+    CompileOptions unpacked = o;
+    unpacked.packedRows = 0;
+    return emitHipSource(g, unpacked);
+  }
 
   std::ostringstream s;
   s << "// generated by spnc-hip for SPN '" << g.name << "': " << g.nodes.size() << " nodes, " << F << " features\n";
@@ -801,6 +1207,26 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     s << "}\n";
   }
 
+  if (waveTile) {
+    // Four values, each saturated (at 255, or with packed rows at the longest table's length: either is outside every
+    // table), into the four bytes of a register: one instruction per value (a minimum whose result goes into one byte
+    // of the destination and leaves the others alone). On this hardware a vector instruction must not read a register
+    // in the cycle after an instruction wrote part of it (the compiler's hazard pass, which does not look into assembler
+    // statements, keeps one wait state between the two): two registers are packed in turns, or idle cycles put between.
+    const std::string sat = std::to_string(e.packedRows ? e.packedSaturation() : 255u) + "u";
+    auto one = [](const char* dst, unsigned src, unsigned byte, unsigned satOperand) {
+      return std::string("v_min_u32_sdwa ") + dst + ", %" + std::to_string(src) + ", %" + std::to_string(satOperand) + " dst_sel:BYTE_" + std::to_string(byte) +
+             " dst_unused:" + (byte ? "UNUSED_PRESERVE" : "UNUSED_PAD") + " src0_sel:DWORD src1_sel:DWORD\\n\\t";
+    };
+    s << "static __device__ __forceinline__ unsigned spn_pack4(unsigned a, unsigned b, unsigned c, unsigned d) {\n  unsigned q;\n  asm(\"";
+    for (unsigned k = 0; k < 4; ++k) s << one("%0", 1 + k, k, 5) << "s_nop 0" << (k < 3 ? "\\n\\t" : "");
+    s << "\"\n      : \"=&v\"(q) : \"v\"(a), \"v\"(b), \"v\"(c), \"v\"(d), \"s\"(" << sat << "));\n  return q;\n}\n";
+    s << "static __device__ __forceinline__ void spn_pack8(unsigned& p, unsigned& q, unsigned a0, unsigned a1, unsigned a2, unsigned a3, unsigned b0, unsigned b1, "
+         "unsigned b2, unsigned b3) {\n  asm(\"";
+    for (unsigned k = 0; k < 4; ++k) s << one("%0", 2 + k, k, 10) << one("%1", 6 + k, k, 10);
+    s << "s_nop 0\"\n      : \"=&v\"(p), \"=&v\"(q) : \"v\"(a0), \"v\"(a1), \"v\"(a2), \"v\"(a3), \"v\"(b0), \"v\"(b1), \"v\"(b2), \"v\"(b3), \"s\"(" << sat
+      << "));\n}\n";
+  }
   if (e.vectorRows) {
     s << "static __device__ __forceinline__ void spn_load_row(const feat_t* __restrict__ in, unsigned long long i, feat_t (&x)[SPN_F]) {\n";
     if (vw == 1) {
@@ -821,14 +1247,27 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     s << "}\n";
   }
 
+  // Software pipeline of the transposed load: a wavefront fetches its next tile while it evaluates the current one, in
+  // two halves that turn round in the middle of the kernel body, so that only half a tile of loaded vectors is in
+  // registers at any time. With two wavefronts per SIMD, which is what the tables and registers of such kernels leave
+  // room for, nothing else overlaps memory latency with arithmetic.
+  const bool prefetch = waveTile && e.packedRows && o.prefetchRows != 0 && F >= 8;
+  e.midpointHook = prefetch;
   emitBody();
-  if (e.vectorRows)
+  if (prefetch)
+    s << "template <typename Mid>\nstatic __device__ __forceinline__ real_t spn_eval(const unsigned (&R)[SPN_F / 4], const real_t* __restrict__ tab, Mid&& spn_mid) {\n";
+  else if (e.packedRows)
+    s << "static __device__ __forceinline__ real_t spn_eval(const unsigned (&R)[SPN_F / 4], const real_t* __restrict__ tab) {\n";
+  else if (e.vectorRows)
     s << "static __device__ __forceinline__ real_t spn_eval(const feat_t (&x)[SPN_F], const real_t* __restrict__ tab) {\n";
   else
     s << "static __device__ __forceinline__ real_t spn_eval(const feat_t* __restrict__ row, const real_t* __restrict__ tab) {\n";
   s << e.body.str();
   std::string root = Emitter::v(g.root());
-  if (!e.logSpace) s << "  return spn_log(" << root << ");\n";
+  if (e.packedRows) {
+    s << "  const real_t spn_root = " << root << (e.log2Dom ? (e.f64 ? " * 0x1.62e42fefa39efp-1" : " * 0x1.62e43p-1f") : "") << ";\n"
+      << "  return outside ? " << e.lit(-INFINITY) << " : spn_root;\n";
+  } else if (!e.logSpace) s << "  return spn_log(" << root << ");\n";
   else if (e.log2Dom) s << "  return " << root << (e.f64 ? " * 0x1.62e42fefa39efp-1;\n" : " * 0x1.62e43p-1f;\n");  // back to natural log: * ln 2
   else s << "  return " << root << ";\n";
   s << "}\n";
@@ -884,7 +1323,72 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   if (staged)
     s << "  typedef unsigned int spn_v4 __attribute__((ext_vector_type(4)));\n"
          "  __shared__ __attribute__((aligned(16))) feat_t spn_tile[SPN_BLOCK * SPN_U * SPN_F];\n";
-  s << "  for (unsigned long long base = blockIdx.x * tile; base < n; base += gridDim.x * tile) {\n";
+  if (prefetch) {
+    // r[0 .. count) = pieces `from` .. of the tile at src; and: those pieces packed into the wavefront's LDS buffer.
+    auto issue = [&](unsigned from, unsigned count, const char* indent) {
+      for (unsigned j = 0; j < count; ++j) s << indent << "r[" << j << "] = SPN_LOAD_TILE(src + " << (from + j) * 64 << "u + lane);\n";
+      s << indent << "asm volatile(\"\" ::: \"memory\");\n" << indent << "__builtin_amdgcn_sched_barrier(0);\n";  // the loads are issued here and nowhere later
+    };
+    auto stash = [&](unsigned from, unsigned count, const char* indent) {
+      s << indent << "{\n" << indent << "  unsigned packed[" << count << "];\n";
+      for (unsigned j = 0; j + 1 < count; j += 2)
+        s << indent << "  spn_pack8(packed[" << j << "], packed[" << j + 1 << "], r[" << j << "][0], r[" << j << "][1], r[" << j << "][2], r[" << j << "][3], r[" << j + 1
+          << "][0], r[" << j + 1 << "][1], r[" << j + 1 << "][2], r[" << j + 1 << "][3]);\n";
+      if (count & 1) s << indent << "  packed[" << count - 1 << "] = spn_pack4(r[" << count - 1 << "][0], r[" << count - 1 << "][1], r[" << count - 1 << "][2], r[" << count - 1 << "][3]);\n";
+      for (unsigned j = 0; j < count; ++j)
+        s << indent << "  { const unsigned p = " << (from + j) * 64 << "u + lane; mine[p + p / SPN_Q * (SPN_S - SPN_Q)] = packed[" << j << "]; }\n";
+      s << indent << "}\n";
+    };
+    const unsigned Q = F / 4, H = (Q + 1) / 2;
+    // Piece p = 64 j + lane of a tile (16 bytes, four features of row p / Q) goes to packed dword p of the buffer; row r's
+    // packed dwords r Q .. r Q + Q - 1 sit at stride S. A wavefront's LDS operations complete in order and no other
+    // wavefront touches its buffer, so no barrier is needed. Where there is no full tile to fetch (the batch's end),
+    // the batch's first tile is fetched instead and never used: the loads and their uses then need no branches, which
+    // keeps them where they are written.
+    s << "  const unsigned long long step = gridDim.x * tile;\n"
+         "  const bool big = n >= 64;   // smaller batches have no full tile at all, and nothing is prefetched\n"
+         "  const spn_v4* const tile0 = reinterpret_cast<const spn_v4*>(in);\n"
+         "  spn_v4 r[" << H << "];   // half a tile as loaded: piece 64 j + lane\n"
+         "  if (big) {\n"
+         "    const unsigned long long first = blockIdx.x * tile + (threadIdx.x & ~63u);\n"
+         "    const spn_v4* src = first + 64 <= n ? reinterpret_cast<const spn_v4*>(in + first * SPN_F) : tile0;\n";
+    issue(0, H, "    ");
+    stash(0, H, "    ");
+    issue(H, Q - H, "    ");
+    stash(H, Q - H, "    ");
+    s << "  }\n"
+         "  for (unsigned long long base = blockIdx.x * tile; base < n; base += step) {\n"
+         "    const unsigned long long first = base + (threadIdx.x & ~63u);   // first row of this wavefront's 64\n"
+         "    unsigned R[SPN_Q];   // the lane's row, four features to a register, a byte each\n"
+         "    const unsigned long long i = first + lane;\n"
+         "    if (first + 64 <= n) {\n"
+         "#pragma unroll\n"
+         "      for (unsigned c = 0; c < SPN_Q; ++c) R[c] = mine[lane * SPN_S + c];\n"
+         "    } else {\n"
+         "      // the batch's last, partial group of 64 rows: every lane fetches its own row (idle lanes the last one)\n"
+         "      feat_t x[SPN_F];\n"
+         "      spn_load_row(in, i < n ? i : n - 1, x);\n"
+         "#pragma unroll\n"
+         "      for (unsigned c = 0; c + 1 < SPN_Q; c += 2) spn_pack8(R[c], R[c + 1], x[4 * c], x[4 * c + 1], x[4 * c + 2], x[4 * c + 3], x[4 * c + 4], x[4 * c + 5], x[4 * c + 6], x[4 * c + 7]);\n"
+         "      if (SPN_Q & 1) R[SPN_Q - 1] = spn_pack4(x[SPN_F - 4], x[SPN_F - 3], x[SPN_F - 2], x[SPN_F - 1]);\n"
+         "    }\n"
+         "    const spn_v4* src = first + step + 64 <= n ? reinterpret_cast<const spn_v4*>(in + (first + step) * SPN_F) : tile0;\n"
+         "    if (big) {\n";
+    issue(0, H, "      ");
+    s << "    }\n"
+         "    const real_t value = spn_eval(R, tab, [&] {\n"
+         "      if (big) {\n";
+    stash(0, H, "        ");
+    issue(H, Q - H, "        ");
+    s << "      }\n"
+         "    });\n"
+         "    if (big) {\n";
+    stash(H, Q - H, "      ");
+    s << "    }\n"
+         "    if (i < n) __builtin_nontemporal_store(value, out + i);\n";
+  } else {
+    s << "  for (unsigned long long base = blockIdx.x * tile; base < n; base += gridDim.x * tile) {\n";
+  }
   const char* tail =
       "      for (int u = 0; u < SPN_U; ++u) {\n"
       "        const unsigned long long i = base + (unsigned long long)u * SPN_BLOCK + threadIdx.x;\n"
@@ -894,36 +1398,50 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
       "          out[i] = spn_eval(x, tab);\n"
       "        }\n"
       "      }\n";
-  if (waveTile) {
+  if (prefetch) {
+    // emitted above
+  } else if (waveTile) {
     // Piece p = 64 j + lane of the tile (16 bytes, four features of row p / Q) goes to packed dword p of the tile; row r's
     // packed dwords r Q .. r Q + Q - 1 sit at stride S. A wavefront's LDS operations complete in order and no other
     // wavefront touches its buffer, so no barrier is needed.
     s << "    const unsigned long long first = base + (threadIdx.x & ~63u);   // first row of this wavefront's 64\n"
-         "    feat_t x[SPN_F];\n"
+         "    unsigned R[SPN_Q];   // the lane's row, four features to a register, a byte each\n"
          "    unsigned long long i = first + lane;\n"
          "    if (first + 64 <= n) {\n"
          "      const spn_v4* src = reinterpret_cast<const spn_v4*>(in + first * SPN_F);\n"
          "      spn_v4 r[SPN_Q];\n"
          "#pragma unroll\n"
          "      for (unsigned j = 0; j < SPN_Q; ++j) r[j] = SPN_LOAD_TILE(src + j * 64 + lane);\n"
+      << "      unsigned packed[SPN_Q];\n"
+         "#pragma unroll\n"
+         "      for (unsigned j = 0; j + 1 < SPN_Q; j += 2) spn_pack8(packed[j], packed[j + 1], r[j][0], r[j][1], r[j][2], r[j][3], r[j + 1][0], r[j + 1][1], r[j + 1][2], r[j + 1][3]);\n"
+         "      if (SPN_Q & 1) packed[SPN_Q - 1] = spn_pack4(r[SPN_Q - 1][0], r[SPN_Q - 1][1], r[SPN_Q - 1][2], r[SPN_Q - 1][3]);\n"
          "#pragma unroll\n"
          "      for (unsigned j = 0; j < SPN_Q; ++j) {\n"
-         "        const unsigned a = r[j][0] < 255u ? r[j][0] : 255u, b = r[j][1] < 255u ? r[j][1] : 255u;\n"
-         "        const unsigned c = r[j][2] < 255u ? r[j][2] : 255u, d = r[j][3] < 255u ? r[j][3] : 255u;\n"
          "        const unsigned p = j * 64 + lane;\n"
-         "        mine[p + p / SPN_Q * (SPN_S - SPN_Q)] = a | (b << 8) | (c << 16) | (d << 24);\n"
+         "        mine[p + p / SPN_Q * (SPN_S - SPN_Q)] = packed[j];\n"
          "      }\n"
          "#pragma unroll\n"
-         "      for (unsigned c = 0; c < SPN_Q; ++c) {\n"
-         "        const unsigned q = mine[lane * SPN_S + c];\n"
-         "        x[4 * c] = q & 255u;\n        x[4 * c + 1] = (q >> 8) & 255u;\n        x[4 * c + 2] = (q >> 16) & 255u;\n        x[4 * c + 3] = q >> 24;\n"
-         "      }\n"
+         "      for (unsigned c = 0; c < SPN_Q; ++c) R[c] = mine[lane * SPN_S + c];\n"
          "    } else {\n"
          "      // the batch's last, partial group of 64 rows: every lane fetches its own row (idle lanes the last one)\n"
+         "      feat_t x[SPN_F];\n"
          "      spn_load_row(in, i < n ? i : n - 1, x);\n"
-         "    }\n"
-         "    const real_t value = spn_eval(x, tab);\n"
-         "    if (i < n) __builtin_nontemporal_store(value, out + i);\n";
+         "#pragma unroll\n"
+         "      for (unsigned c = 0; c + 1 < SPN_Q; c += 2) spn_pack8(R[c], R[c + 1], x[4 * c], x[4 * c + 1], x[4 * c + 2], x[4 * c + 3], x[4 * c + 4], x[4 * c + 5], x[4 * c + 6], x[4 * c + 7]);\n"
+         "      if (SPN_Q & 1) R[SPN_Q - 1] = spn_pack4(x[SPN_F - 4], x[SPN_F - 3], x[SPN_F - 2], x[SPN_F - 1]);\n"
+         "    }\n";
+    if (e.packedRows) {
+      s << "    const real_t value = spn_eval(R, tab);\n";
+    } else {
+      s << "    feat_t x[SPN_F];\n"
+           "#pragma unroll\n"
+           "    for (unsigned c = 0; c < SPN_Q; ++c) {\n"
+           "      x[4 * c] = R[c] & 255u;\n      x[4 * c + 1] = (R[c] >> 8) & 255u;\n      x[4 * c + 2] = (R[c] >> 16) & 255u;\n      x[4 * c + 3] = R[c] >> 24;\n"
+           "    }\n"
+           "    const real_t value = spn_eval(x, tab);\n";
+    }
+    s << "    if (i < n) __builtin_nontemporal_store(value, out + i);\n";
   } else if (staged) {
     s << "    if (base + tile <= n) {\n"
          "      const spn_v4* src = reinterpret_cast<const spn_v4*>(in + base * SPN_F);\n"

@@ -25,6 +25,7 @@ struct JitSource {
   bool doubleConstants = false;  // computes in double: constants live in registers, not in instruction literals
   bool oneTilePerBlock = false;
   bool waveTransposedInput = false;  // every wavefront copies its 64 rows with coalesced loads, packed to bytes, through its own LDS buffer
+  bool packedRows = false;    // the kernel body works on rows packed to a byte per feature (sibling products evaluated together)
   bool stagedInput = false;   // rows reach the lanes through an LDS tile ("gpu-shared-mem")
 };
 

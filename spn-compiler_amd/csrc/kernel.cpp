@@ -60,6 +60,25 @@ std::vector<char> compileWithHipRtc(const JitSource& js, int optLevel, int machi
   return code;
 }
 
+// Registers the compiler spilled to scratch memory, from the code object's metadata (a msgpack map in an ELF note:
+// the key ".vgpr_spill_count" is followed by an unsigned integer). 0 when the key is absent.
+uint32_t spilledRegisters(const std::vector<char>& code) {
+  static const char key[] = ".vgpr_spill_count";
+  const size_t keyLen = sizeof(key) - 1;
+  uint32_t most = 0;
+  for (size_t at = 0; at + keyLen + 5 <= code.size(); ++at) {
+    if (std::memcmp(code.data() + at, key, keyLen) != 0) continue;
+    const unsigned char* v = reinterpret_cast<const unsigned char*>(code.data()) + at + keyLen;
+    uint32_t n = 0;
+    if (v[0] < 0x80) n = v[0];
+    else if (v[0] == 0xcc) n = v[1];
+    else if (v[0] == 0xcd) n = (uint32_t(v[1]) << 8) | v[2];
+    else if (v[0] == 0xce) n = (uint32_t(v[1]) << 24) | (uint32_t(v[2]) << 16) | (uint32_t(v[3]) << 8) | v[4];
+    most = std::max(most, n);
+  }
+  return most;
+}
+
 // ---- kernel file: magic, then tagged little-endian fields ----
 const char kMagic[8] = {'S', 'P', 'N', 'C', 'H', 'I', 'P', 2};
 
@@ -265,6 +284,15 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
     // about 7x slower on the 16-feature Gaussian tree).
     const int level = (js.libraryMath && !o.optLevelGiven) ? 1 : o.optLevel;
     k->codeObject_ = compileWithHipRtc(js, level, o.machineLicm);
+    if (js.packedRows && o.packedRows < 0 && spilledRegisters(k->codeObject_) > 0) {
+      // Packed rows keep one or two values per small-domain feature in registers for the whole kernel; on graphs
+      // where that does not fit (measured: 2640 nodes, 537 spilled registers, 6.9 ms against 1.1 ms) the kernel
+      // with one index per feature is built instead.
+      CompileOptions unpacked = o;
+      unpacked.packedRows = 0;
+      js = emitHipSource(g, unpacked);
+      k->codeObject_ = compileWithHipRtc(js, level, o.machineLicm);
+    }
     k->entry_ = js.entry;
     k->blockSize_ = js.blockSize;
     k->samplesPerLane_ = js.samplesPerLane;

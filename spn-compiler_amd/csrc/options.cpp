@@ -94,6 +94,18 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       if (o.samplesPerLane < 0 || o.samplesPerLane > 16) throw std::runtime_error("hip-samples-per-lane must be in [0,16]");
     } else if (key == "hip-jit-max-ops") {
       o.jitMaxOps = parseInt(key, val);
+    } else if (key == "hip-prefetch-rows") {
+      o.prefetchRows = parseBool(val) ? 1 : 0;
+    } else if (key == "hip-hoist-feature-values") {
+      o.hoistFeatureValues = parseBool(val);
+    } else if (key == "hip-packed-rows") {
+      o.packedRows = parseBool(val) ? 1 : 0;
+    } else if (key == "hip-one-hot-max-domain") {
+      o.oneHotMaxDomain = parseInt(key, val);
+      if (o.oneHotMaxDomain < 0 || o.oneHotMaxDomain > 16) throw std::runtime_error("hip-one-hot-max-domain must be in [0,16]");
+    } else if (key == "hip-fused-batch") {
+      o.fusedBatch = parseInt(key, val);
+      if (o.fusedBatch < 0 || o.fusedBatch > 16) throw std::runtime_error("hip-fused-batch must be in [0,16]");
     } else if (key == "hip-wave-transpose") {
       o.waveTranspose = parseBool(val) ? 1 : 0;
     } else if (key == "hip-nontemporal-loads") {
@@ -133,6 +145,7 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       o.inlineMath = val == "auto" ? -1 : (parseBool(val) ? 1 : 0);
     } else if (key == "hip-table-budget-kib") {
       o.tableBudgetKiB = parseInt(key, val);
+      o.tableBudgetGiven = true;
       if (o.tableBudgetKiB < 0 || o.tableBudgetKiB > 140) throw std::runtime_error("hip-table-budget-kib must be in [0,140]");
     } else if (key == "hip-joint-max-entries") {
       o.jointMaxEntries = parseInt(key, val);

@@ -41,6 +41,7 @@ struct CompileOptions {
   int tableGroupWindow = 96;                   // "hip-table-group-window": tables of a group are used within this many table uses of each other
   int tablePadKiB = 18;                        // "hip-table-pad-kib": LDS beyond the table budget that blocks of four columns may take (unused columns)
   int tableBudgetKiB = 62;                     // "hip-table-budget-kib": LDS the table pool may grow to when leaves are paired into joint tables
+  bool tableBudgetGiven = false;               // without the option, kernels on packed rows pair up to 80 KiB (measured on the 100-feature discrete graph: 0.75 ms against 0.78 ms at 62 KiB)
   int jointMaxEntries = 160;                   // "hip-joint-max-entries": largest joint table (entries) a pair of table leaves may get
   int interpShortSlots = 0;                    // "hip-interp-short-slots": LDS value slots per lane the interpreter program aims for (0 = automatic)
   bool interpLeafRegions = true;               // "hip-interp-leaf-regions": Gaussian leaf products read by one matrix-form outer sum are computed inside it
@@ -51,6 +52,11 @@ struct CompileOptions {
   int interpLdsSlots = 0;                      // "hip-interp-lds-slots": upper bound on the value slots the launcher keeps in LDS (0 = automatic)
   int interpStagedLong = -1;                   // "hip-interp-staged-features": lds|spill (-1 = automatic): tier of the staged input features
   long interpLongRange = -1;                   // "hip-interp-long-range": values living longer than this many instructions go to the long-lived pool (-1 = automatic)
+  int packedRows = -1;                         // "hip-packed-rows": wide rows of small integer features stay packed four to a register and the table leaves of sibling products are evaluated together (1), not (0), decided per kernel (-1)
+  int oneHotMaxDomain = 3;                     // "hip-one-hot-max-domain": with packed rows, table leaves over at most this many categories are evaluated as multiply-adds on the vector unit instead of LDS reads
+  int prefetchRows = -1;                       // "hip-prefetch-rows": with the per-wavefront transposed load, the loads of a wavefront's next 64 rows are issued before the current ones are evaluated and stay in registers meanwhile (-1 = with packed rows)
+  bool hoistFeatureValues = true;              // "hip-hoist-feature-values": with packed rows, the values (and squares) of the features whose leaves are polynomials are computed once at the top of the kernel (false = again in every group of products that uses them: more arithmetic, fewer registers)
+  int fusedBatch = -1;                         // "hip-fused-batch": with packed rows, LDS reads of this many table units are issued before the values of the batch before are added (0 = every unit on its own, no scheduling barriers; -1 = 2 when rows are prefetched, which leaves fewer registers, else 4)
   int waveTranspose = -1;                       // "hip-wave-transpose": rows of 32-bit integer features reach the lanes through a per-wave LDS transpose of packed bytes (1), not (0), decided per kernel (-1)
   int minBlocksPerCU = 0;                      // "hip-min-blocks-per-cu": register budget hint for the generated kernel (0 = none)
   int blocksPerCU = 0;                         // "hip-blocks-per-cu": 0 = resident blocks (persistent), -1 = one tile per block, n = n per CU

@@ -296,6 +296,33 @@ Graph buildGraph(const RawQuery& q) {
   uint32_t rootIdx = placed.at(defined[m.rootNode]);
   if (rootIdx != g.nodes.size() - 1) fatal("internal error: root is not last in schedule");
 
+  // Scopes, children first: completeness and decomposability.
+  {
+    const size_t words = (g.numFeatures + 63) / 64;
+    std::vector<std::vector<uint64_t>> scope(g.nodes.size(), std::vector<uint64_t>(words, 0));
+    bool ok = true;
+    for (size_t i = 0; i < g.nodes.size() && ok; ++i) {
+      const GraphNode& n = g.nodes[i];
+      if (n.kind != NodeKind::Product && n.kind != NodeKind::Sum) {
+        scope[i][n.feature / 64] |= uint64_t(1) << (n.feature % 64);
+        continue;
+      }
+      for (size_t k = 0; k < n.children.size() && ok; ++k) {
+        const std::vector<uint64_t>& cs = scope[n.children[k]];
+        if (n.kind == NodeKind::Sum) {
+          if (k == 0) scope[i] = cs;
+          else if (scope[i] != cs) ok = false;
+        } else {
+          for (size_t w = 0; w < words; ++w) {
+            if (scope[i][w] & cs[w]) ok = false;
+            scope[i][w] |= cs[w];
+          }
+        }
+      }
+    }
+    g.completeDecomposable = ok;
+  }
+
   // Use counts and statistics.
   for (auto& n : g.nodes)
     for (uint32_t c : n.children) g.nodes[c].uses++;

@@ -114,6 +114,10 @@ struct Graph {
   int32_t batchSize = 1;
   std::vector<GraphNode> nodes;  // children first; root is nodes.back()
   GraphStats stats;
+  // Complete and decomposable: the children of every sum cover the same features, those of every product disjoint
+  // ones. Then an input outside a table leaf's range makes the root's value log 0 whatever else the graph computes,
+  // because every path from the root meets a leaf of that feature (what the kernels may rely on for such inputs).
+  bool completeDecomposable = false;
   uint32_t root() const { return uint32_t(nodes.size() - 1); }
 };
 

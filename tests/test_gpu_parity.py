@@ -169,7 +169,7 @@ def test_grouped_tables_on_the_discrete_configuration(native, variant, cfg):
     spn, X = c["spn"](), c["inputs"](4099)
     X[5, :] = 77            # out of every feature's range
     X[6, 3] = 9
-    k = compile_spn(native, spn, c["dtype"], marginal=False, **GROUPED[variant])
+    k = compile_spn(native, spn, c["dtype"], marginal=False, **GROUPED[variant], **{"hip-packed-rows": "false"})
     src = k.source()
     grouped = variant not in ("plain", "no-room", "small-pool", "float64")
     if cfg == "c3":   # products of up to fifty leaves: which layout the generator picks is its own business, the values count
@@ -185,6 +185,55 @@ def test_grouped_tables_on_the_discrete_configuration(native, variant, cfg):
     else:
         check_f32(got, m, X, False)
         assert np.isneginf(got[5]) and np.isneginf(got[6])
+
+
+PACKED = {
+    "default": {},                                        # rows packed to bytes, sibling products fused, one-hot leaves up to 3 categories
+    "unbatched": {"hip-fused-batch": 0},
+    "batch-7": {"hip-fused-batch": 7},
+    "all-lds": {"hip-one-hot-max-domain": 0},
+    "one-hot-5": {"hip-one-hot-max-domain": 5},
+    "no-joint": {"hip-joint-tables": "false"},
+    "small-budget": {"hip-table-budget-kib": 24},         # pairs are split again until the tables fit
+    "float64": {"hip-compute-type": "float64"},
+    "block-256": {"hip-block-size": 256},
+    "per-lane-rows": {"hip-wave-transpose": "false"},     # no per-wavefront transposed load: rows stay unpacked
+}
+
+
+@pytest.mark.parametrize("cfg", ["c3", "c3_deep"])
+@pytest.mark.parametrize("variant", sorted(PACKED))
+def test_packed_rows_on_the_discrete_configuration(native, variant, cfg):
+    """Wide rows of small integers kept four features to a register, the table leaves of sibling products evaluated
+    together (joint tables over pairs of features, one-hot multiply-adds for small domains): every variant gives the
+    oracle's values, inputs outside a feature's range included (they make the result log 0)."""
+    from spnc import synthetic as syn
+    c = syn.CONFIGS[cfg]
+    spn, X = c["spn"](), c["inputs"](4099)
+    X[5, :] = 77            # out of every feature's range
+    X[6, 3] = 9             # out of one feature's range
+    X[7, 97] = 2 ** 31 - 1  # far out (a feature of the last register)
+    X[8, 0] = 255
+    X[9, 1] = 256           # does not fit a byte
+    # Left to itself the compiler drops packed rows when the kernel spills registers (the deeper graph does): the
+    # variants ask for them outright, "default" leaves the choice to the compiler.
+    opts = dict(PACKED[variant])
+    if variant != "default":
+        opts.setdefault("hip-packed-rows", "true")
+    k = compile_spn(native, spn, c["dtype"], marginal=False, **opts)
+    src = k.source()
+    packed = "unsigned PK0 = R[0]" in src and "spn_rows" in src
+    assert packed == (variant != "per-lane-rows" and not (variant == "default" and cfg == "c3_deep"))
+    got = run(k, X)
+    m = oracle_model(spn, c["dtype"])
+    if variant == "float64":
+        assert got.dtype == np.float64
+        ref = ev.ll_closed_f64(m, X, marginal=False)
+        assert np.array_equal(np.isneginf(got), np.isneginf(ref))
+        assert np.abs(got[np.isfinite(ref)] - ref[np.isfinite(ref)]).max() <= F64_TOL
+    else:
+        check_f32(got, m, X, False)
+    assert all(np.isneginf(got[r]) for r in (5, 6, 7, 8, 9)) and np.isfinite(got[10])
 
 
 @pytest.mark.parametrize("dtype,marginal", [("uint8", False), ("int32", False), ("float32", True), ("float64", True)])
