@@ -58,6 +58,8 @@ typedef struct spnc_hip_info {
   unsigned feature_is_float; /* 1: inputs are IEEE floats of bytes_per_feature bytes; 0: unsigned integers of that width (signed
                                 integer arrays of the same width are read as unsigned, as the reference's index_cast / uitofp do) */
   unsigned support_marginal; /* the query was compiled with NaN-marginalisation */
+  unsigned num_tasks;        /* kernels one execution launches: 1, or the tasks a graph was cut into by "maxTaskSize" */
+  unsigned task_rows;        /* rows of intermediate values that pass between those tasks (each as long as the batch) */
 } spnc_hip_info;
 
 /* spn_compiler::isTargetSupported("HIP") (compiler/src/Driver.cpp:47-59): 1 if a gfx950 device

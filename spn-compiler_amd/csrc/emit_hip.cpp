@@ -880,8 +880,11 @@ struct Emitter {
     if (emitted[i]) return;
     emitted[i] = true;
     const auto& n = g.nodes[i];
-    if (n.kind != NodeKind::Product && n.kind != NodeKind::Sum) emitFeaturePrep(n.feature);
+    if (n.kind != NodeKind::Product && n.kind != NodeKind::Sum && n.kind != NodeKind::External) emitFeaturePrep(n.feature);
     switch (n.kind) {
+      case NodeKind::External:  // computed by an earlier task: row `feature` of the intermediate buffer, this sample's column
+        body << "  const real_t " << v(i) << " = spn_in[" << n.feature << "ull * spn_n];\n";
+        break;
       case NodeKind::Gaussian: {
         // log: coef + (x-mean)^2 * den with coef = -ln(sd) - ln(2 pi)/2, den = -1/(2 sd^2)
         // (mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:306-374); linear: coef' * exp((x-mean)^2 * den)
@@ -1012,7 +1015,7 @@ unsigned pickVectorBytes(unsigned rowBytes, unsigned elemBytes) {
 
 }  // namespace
 
-JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
+JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::string& entry) {
   Emitter e(g, o);
   // Short rows are fetched with the widest vector loads their size allows, all samples of a
   // lane up front; wide rows are read feature by feature next to the first use.
@@ -1021,7 +1024,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     // Packed rows: wide rows of 32-bit integers that only feed table leaves with short tables, in a complete and
     // decomposable graph (an input outside a one-hot feature's range is reported through a flag, not through a table).
     bool eligible = e.logSpace && e.vectorRows && !g.ftype.isFloat && g.ftype.bytes == 4 && g.numFeatures % 4 == 0 &&
-                    g.numFeatures * 4 >= 128 && g.completeDecomposable && !g.supportMarginal && o.samplesPerLane <= 1;
+                    g.numFeatures * 4 >= 128 && g.completeDecomposable && !g.supportMarginal && o.samplesPerLane <= 1 && !g.isTask;
     bool anyTable = false;
     for (const auto& n : g.nodes) {
       if (n.kind == NodeKind::Gaussian) eligible = false;
@@ -1034,7 +1037,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   }
   e.prepare();
   JitSource js;
-  js.entry = "spn_kernel";
+  js.entry = entry;
   js.blockSize = o.blockSize ? unsigned(o.blockSize) : 256u;
   // Grouped tables with packed indices leave the kernel at about 140 registers and take up to 80 KiB of LDS: one
   // block of 1024 threads per CU then runs four waves per SIMD on one copy of the tables (C3: 1.19 ms with two
@@ -1062,6 +1065,13 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
       for (uint32_t f = 0; f < F; ++f)
         if (e.featUsed[f] && e.featTableLen[f]) e.emitFeaturePrep(f);
     if (e.packedIndices) e.emitPackedIndices();
+    if (g.isTask) {
+      for (uint32_t node : g.taskOutputs) e.emitNode(node);
+      if (g.taskFinal) e.emitNode(g.root());
+      for (size_t k = 0; k < g.taskOutputs.size(); ++k)
+        e.body << "  spn_res[" << g.taskOutputSlots[k] << "ull * spn_n] = " << Emitter::v(g.taskOutputs[k]) << ";\n";
+      return;
+    }
     e.emitNode(g.root());
   };
   const unsigned vb = e.vectorRows ? pickVectorBytes(rowBytes, eb) : eb;
@@ -1073,7 +1083,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   const size_t work = g.nodes.size() + g.stats.sumTerms;
   unsigned U = unsigned(o.samplesPerLane);
   if (U == 0) U = (work <= 4000 && !g.supportMarginal && size_t(js.tableEntries) * realBytes <= 16 * 1024) ? 2 : 1;
-  if (!e.vectorRows || e.packedRows) U = 1;
+  if (!e.vectorRows || e.packedRows || g.isTask) U = 1;  // tasks: one sample per lane, rows fetched by their lane
   js.samplesPerLane = U;
   // Kernels that sit on the HBM bound and stage their input tile through LDS run 2-3 % faster with
   // 512-thread blocks (measured on the six-feature product: 0.82 against 0.80 of the HBM peak).
@@ -1094,7 +1104,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   bool waveTile = false;
   unsigned waveStride = 0;  // dwords per packed row in LDS: odd, so that the 64 lanes' reads fall into distinct banks
   {
-    bool eligible = e.vectorRows && !g.ftype.isFloat && eb == 4 && F % 4 == 0 && U == 1 && rowBytes >= 128;
+    bool eligible = e.vectorRows && !g.ftype.isFloat && eb == 4 && F % 4 == 0 && U == 1 && rowBytes >= 128 && !g.isTask;
     for (uint32_t f = 0; f < F && eligible; ++f)
       if (e.featGauss[f] || e.featTableLen[f] > 255) eligible = false;
     if (eligible && (o.waveTranspose == 1 || (e.packedRows && o.waveTranspose != 0))) {  // beside unpacked indices it gains nothing (0.79 against 0.78 ms on the 100-feature discrete graph): only with packed rows, or on request
@@ -1113,7 +1123,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   if (e.packedRows && !waveTile) {  // the row buffers do not fit beside the tables: the same kernel with unpacked rows
     CompileOptions unpacked = o;
     unpacked.packedRows = 0;
-    return emitHipSource(g, unpacked);
+    return emitHipSource(g, unpacked, entry);
   }
 
   std::ostringstream s;
@@ -1252,6 +1262,10 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   // registers at any time. With two wavefronts per SIMD, which is what the tables and registers of such kernels leave
   // room for, nothing else overlaps memory latency with arithmetic.
   const bool prefetch = waveTile && e.packedRows && o.prefetchRows != 0 && F >= 8;
+  // A task reads the values of earlier tasks from, and writes its own results to, the column of its sample in the
+  // intermediate buffer (spn_in and spn_res point at that column; its rows are spn_n values apart).
+  const char* taskParams = g.isTask ? ", const real_t* __restrict__ spn_in, real_t* __restrict__ spn_res, unsigned long long spn_n" : "";
+  const char* taskArgs = g.isTask ? ", ext + i, res + i, n" : "";
   e.midpointHook = prefetch;
   emitBody();
   if (prefetch)
@@ -1259,15 +1273,16 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   else if (e.packedRows)
     s << "static __device__ __forceinline__ real_t spn_eval(const unsigned (&R)[SPN_F / 4], const real_t* __restrict__ tab) {\n";
   else if (e.vectorRows)
-    s << "static __device__ __forceinline__ real_t spn_eval(const feat_t (&x)[SPN_F], const real_t* __restrict__ tab) {\n";
+    s << "static __device__ __forceinline__ real_t spn_eval(const feat_t (&x)[SPN_F], const real_t* __restrict__ tab" << taskParams << ") {\n";
   else
-    s << "static __device__ __forceinline__ real_t spn_eval(const feat_t* __restrict__ row, const real_t* __restrict__ tab) {\n";
+    s << "static __device__ __forceinline__ real_t spn_eval(const feat_t* __restrict__ row, const real_t* __restrict__ tab" << taskParams << ") {\n";
   s << e.body.str();
   std::string root = Emitter::v(g.root());
   if (e.packedRows) {
     s << "  const real_t spn_root = " << root << (e.log2Dom ? (e.f64 ? " * 0x1.62e42fefa39efp-1" : " * 0x1.62e43p-1f") : "") << ";\n"
       << "  return outside ? " << e.lit(-INFINITY) << " : spn_root;\n";
-  } else if (!e.logSpace) s << "  return spn_log(" << root << ");\n";
+  } else if (g.isTask && !g.taskFinal) s << "  return " << e.lit(0.0) << ";\n";
+  else if (!e.logSpace) s << "  return spn_log(" << root << ");\n";
   else if (e.log2Dom) s << "  return " << root << (e.f64 ? " * 0x1.62e42fefa39efp-1;\n" : " * 0x1.62e43p-1f;\n");  // back to natural log: * ln 2
   else s << "  return " << root << ";\n";
   s << "}\n";
@@ -1283,7 +1298,8 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   if (minBlocks == 0 && (js.blockSize == 1024 || waveTile)) minBlocks = 1;
   if (minBlocks == 0 && js.tablesInLds && ldsTables > 40 * 1024 && ldsTables <= 80 * 1024 && tableFeatures <= 136) minBlocks = 2;
   s << "extern \"C\" __global__ void __launch_bounds__(SPN_BLOCK" << (minBlocks > 0 ? ", " + std::to_string(minBlocks) : std::string()) << ") " << js.entry
-    << "(const feat_t* __restrict__ in, real_t* __restrict__ out, unsigned long long n) {\n";
+    << "(const feat_t* __restrict__ in, real_t* __restrict__ out, unsigned long long n"
+    << (g.isTask ? ", const real_t* __restrict__ ext, real_t* __restrict__ res" : "") << ") {\n";
   if (e.log2Dom && e.f64)
     s << "  for (unsigned t = threadIdx.x; t < 64; t += SPN_BLOCK) spn_exp2_lds[t] = spn_exp2_table[t];\n"
          "  for (unsigned t = threadIdx.x; t < 512; t += SPN_BLOCK) spn_log2_lds[t] = spn_log2_table[t];\n"
@@ -1307,7 +1323,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
   // than to the VALU bound (about 6.4e12 B/s against 6e13 lane-operations/s on MI355X).
   const double tHbm = double(rowBytes + realBytes) / 6.4e12, tValu = double(g.stats.issueSlotsMin()) / 6.0e13;
   const bool wantStaged = o.gpuSharedMem < 0 ? tHbm > 0.5 * tValu : o.gpuSharedMem == 1;
-  const bool staged = !waveTile && wantStaged && e.vectorRows && tileBytes % 16 == 0 && tileBytes + ldsTables <= 64 * 1024;
+  const bool staged = !waveTile && !g.isTask && wantStaged && e.vectorRows && tileBytes % 16 == 0 && tileBytes + ldsTables <= 64 * 1024;
   js.stagedInput = staged;
   // Blocks with next to no set-up take one tile each; blocks that stage tables stay resident.
   js.oneTilePerBlock = js.tableEntries <= 256;
@@ -1467,9 +1483,11 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o) {
     if (e.vectorRows)
       s << "      feat_t x[SPN_F];\n"
            "      spn_load_row(in, i, x);\n"
-           "      __builtin_nontemporal_store(spn_eval(x, tab), out + i);\n";
+           "      const real_t value = spn_eval(x, tab" << taskArgs << ");\n";
     else
-      s << "      __builtin_nontemporal_store(spn_eval(in + i * SPN_F, tab), out + i);\n";
+      s << "      const real_t value = spn_eval(in + i * SPN_F, tab" << taskArgs << ");\n";
+    if (!g.isTask || g.taskFinal) s << "      __builtin_nontemporal_store(value, out + i);\n";
+    else s << "      (void)value;\n";
     s << "    }\n";
   } else {
     s << "    if (base + tile <= n) {\n"

@@ -29,6 +29,8 @@ struct JitSource {
   bool stagedInput = false;   // rows reach the lanes through an LDS tile ("gpu-shared-mem")
 };
 
-JitSource emitHipSource(const Graph& g, const CompileOptions& o);
+// `entry` names the kernel. A task of a partitioned graph (g.isTask) takes two more arguments: the intermediate buffer to
+// read from and to write to, [rows][n] values of the kernel's compute type.
+JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::string& entry = "spn_kernel");
 
 }  // namespace spnc_hip

@@ -80,7 +80,7 @@ uint32_t spilledRegisters(const std::vector<char>& code) {
 }
 
 // ---- kernel file: magic, then tagged little-endian fields ----
-const char kMagic[8] = {'S', 'P', 'N', 'C', 'H', 'I', 'P', 2};
+const char kMagic[8] = {'S', 'P', 'N', 'C', 'H', 'I', 'P', 3};
 
 struct Writer {
   std::vector<char> buf;
@@ -258,10 +258,9 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
   const bool hardwareTranscendentals = o.useLogSpace && o.computeType == ComputeType::F32 && o.log2Domain;
   const uint64_t ops = g.nodes.size() + g.stats.productAdds + g.stats.sumTerms * (hardwareTranscendentals ? 1 : 6);
   // The reference's "maxTaskSize" bounds the operations per compiled task by cutting the graph into several tasks
-  // (mlir/lib/Dialect/LoSPN/Passes/LoSPNTaskPartitioner.cpp:36-148). Here a graph above that bound is not cut:
-  // it goes to the interpreter, whose code size does not depend on the graph.
-  uint64_t jitLimit = uint64_t(std::max(0, o.jitMaxOps));
-  if (o.maxTaskSize > 0) jitLimit = std::min<uint64_t>(jitLimit, uint64_t(o.maxTaskSize));
+  // (mlir/lib/Dialect/LoSPN/Passes/LoSPNTaskPartitioner.cpp:36-148); the straight-line kernels are cut the same way
+  // (partition.cpp). The interpreter's code does not grow with the graph and ignores the option.
+  const uint64_t jitLimit = uint64_t(std::max(0, o.jitMaxOps));
   bool useInterp = o.kernelMode == KernelMode::Interpreter || (o.kernelMode == KernelMode::Auto && ops > jitLimit);
   if (useInterp && !o.useLogSpace) {
     if (o.kernelMode == KernelMode::Interpreter) fatal("COMPILATION ERROR: the interpreter kernel supports log-space computation only");
@@ -277,7 +276,47 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
     k->gridPolicy_ = std::max(0, o.blocksPerCU);  // a limit on the resident blocks; the interpreter is always persistent
   } else {
     k->kind_ = SPNC_HIP_KERNEL_JIT;
-    JitSource js = emitHipSource(g, o);
+    TaskPlan plan;
+    if (o.maxTaskSize > 0) plan = partitionGraph(g, o.maxTaskSize);
+    JitSource js;
+    if (plan.tasks.size() > 1) {
+      // One translation unit with a kernel per task: each task's source in a namespace of its own, the macros it
+      // defines dropped again after it.
+      std::string all;
+      js.inputAlign = 1;
+      // Whether the exp/log routines are inlined is decided by the size of the whole graph, as without the cut: what
+      // costs hipRTC time is the sum of all inlined copies, whichever kernel they land in.
+      CompileOptions taskOptions = o;
+      if (o.inlineMath < 0) taskOptions.inlineMath = g.nodes.size() + g.stats.sumTerms <= 4000 ? 1 : 0;
+      for (size_t t = 0; t < plan.tasks.size(); ++t) {
+        const Graph& tg = plan.tasks[t];
+        JitSource one = emitHipSource(tg, taskOptions, "spn_task" + std::to_string(t));
+        size_t valuesIn = 0;
+        for (const auto& n : tg.nodes) valuesIn += n.kind == NodeKind::External ? 1 : 0;
+        all += "// task " + std::to_string(t) + " of " + std::to_string(plan.tasks.size()) + ": " + std::to_string(taskWeight(tg)) + " operations, " +
+               std::to_string(valuesIn) + " values in, " + std::to_string(tg.taskOutputs.size()) + " values out" + (tg.taskFinal ? ", the result" : "") + "\n";
+        all += "namespace spn_task_scope" + std::to_string(t) + " {\n" + one.source + "}  // task " + std::to_string(t) +
+               "\n#undef SPN_LOAD\n#undef SPN_LOAD_TILE\n#undef SPN_F\n#undef SPN_BLOCK\n#undef SPN_U\n#undef SPN_NTAB\n#undef SPN_DOUBLE_TABLES\n"
+               "#undef SPN_EXP2_TABLE\n#undef SPN_LOG2_TABLE\n#undef SPN_POLY\n";
+        Task task;
+        task.entry = one.entry;
+        task.blockSize = one.blockSize;
+        task.gridPolicy = o.blocksPerCU != 0 ? o.blocksPerCU : (one.oneTilePerBlock ? -1 : 0);
+        k->tasks_.push_back(task);
+        js.inputAlign = std::max(js.inputAlign, one.inputAlign);
+        js.libraryMath = js.libraryMath || one.libraryMath;
+        js.doubleConstants = js.doubleConstants || one.doubleConstants;
+        js.bytesPerResult = one.bytesPerResult;
+      }
+      js.source = std::move(all);
+      js.entry = k->tasks_.back().entry;
+      js.blockSize = k->tasks_.back().blockSize;
+      js.samplesPerLane = 1;
+      k->taskSlots_ = plan.slots;
+      k->taskBufferMiB_ = unsigned(o.taskBufferMiB);
+    } else {
+      js = emitHipSource(g, o);
+    }
     // The generated code is already straight-line and CSE'd. Kernels that inline the library
     // exp/log are built at -O1 unless the caller asks otherwise: at -O2 and above the mid-level
     // optimiser stretches live ranges until the float64 kernels spill (512 VGPRs plus scratch,
@@ -345,6 +384,14 @@ void Kernel::save(const std::string& path) const {
     w.u32(samplesPerLane_);
     w.u32(inputAlign_);
     w.u32(uint32_t(gridPolicy_));
+    w.u32(uint32_t(tasks_.size()));
+    for (const Task& t : tasks_) {
+      w.str(t.entry);
+      w.u32(t.blockSize);
+      w.u32(uint32_t(t.gridPolicy));
+    }
+    w.u32(taskSlots_);
+    w.u32(taskBufferMiB_);
   } else {
     w.u32(prog_.f64);
     w.u32(prog_.log2Domain);
@@ -399,6 +446,17 @@ std::unique_ptr<Kernel> Kernel::load(const std::string& kernelFile) {
     k->samplesPerLane_ = r.u32();
     k->inputAlign_ = r.u32();
     k->gridPolicy_ = int(r.u32());
+    const uint32_t numTasks = r.u32();
+    if (numTasks > (1u << 20)) fatal("RUNTIME ERROR: kernel file " + kernelFile + " is damaged (task count)");
+    for (uint32_t t = 0; t < numTasks; ++t) {
+      Task task;
+      task.entry = r.str();
+      task.blockSize = r.u32();
+      task.gridPolicy = int(r.u32());
+      k->tasks_.push_back(task);
+    }
+    k->taskSlots_ = r.u32();
+    k->taskBufferMiB_ = r.u32();
   } else if (k->kind_ == SPNC_HIP_KERNEL_INTERPRETER) {
     k->prog_.f64 = r.u32() != 0;
     k->prog_.log2Domain = r.u32() != 0;
@@ -438,6 +496,14 @@ std::unique_ptr<Kernel> Kernel::load(const std::string& kernelFile) {
     if (k->inputAlign_ == 0 || k->inputAlign_ > 16 || (k->inputAlign_ & (k->inputAlign_ - 1)) != 0) reject("input alignment");
     if (k->gridPolicy_ < -1 || k->gridPolicy_ > 64) reject("grid policy");
     if (k->entry_.empty() || k->codeObject_.size() < 64) reject("code object");
+    if (k->tasks_.size() == 1 || k->taskSlots_ > (1u << 24) || (k->tasks_.empty() && k->taskSlots_ != 0)) reject("tasks");
+    for (const Task& t : k->tasks_) {
+      if (t.blockSize < 64 || t.blockSize > 1024 || t.blockSize % 64 != 0) reject("block size of a task");
+      if (t.gridPolicy < -1 || t.gridPolicy > 64) reject("grid policy of a task");
+      if (t.entry.empty()) reject("entry point of a task");
+    }
+    if (!k->tasks_.empty() && k->samplesPerLane_ != 1) reject("samples per lane");
+    if (k->taskBufferMiB_ < 1 || k->taskBufferMiB_ > 65536) reject("size of the intermediate buffer");
   } else {
     if (k->bytesPerResult_ != (k->prog_.f64 ? 8u : 4u)) reject("result width");
     checkInterpProgram(k->prog_, k->numFeatures_);
@@ -477,6 +543,8 @@ void Kernel::fillInfo(spnc_hip_info* info) const {
   info->fused_min = stats_.fusedMin;
   info->feature_is_float = featureType_ == unsigned(FeatureType::F32) || featureType_ == unsigned(FeatureType::F64);
   info->support_marginal = marginal_ ? 1u : 0u;
+  info->num_tasks = tasks_.empty() ? 1u : unsigned(tasks_.size());
+  info->task_rows = taskSlots_;
 }
 
 void Kernel::ensureDevice() {
@@ -563,6 +631,12 @@ void Kernel::prepareDevice() {
     int nb = 0;
     hipCheck(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&nb, function_, int(blockSize_), 0), "occupancy query");
     blocksPerCU_ = std::max(1, nb);
+    for (Task& t : tasks_) {
+      hipCheck(hipModuleGetFunction(&t.function, module_, t.entry.c_str()), "hipModuleGetFunction");
+      hipCheck(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&nb, t.function, int(t.blockSize), 0), "occupancy query");
+      t.blocksPerCU = std::max(1, nb);
+    }
+    if (!tasks_.empty()) hipCheck(hipEventCreateWithFlags(&interDone_, hipEventDisableTiming), "hipEventCreate");
   } else {
     const size_t rb = prog_.f64 ? 8 : 4;
     buildImages();
@@ -603,9 +677,16 @@ void Kernel::releaseDevice() {
   dTables_ = nullptr;
   dStaged_ = nullptr;
   dSpill_ = nullptr;
+  if (dInter_) (void)hipFree(dInter_);
+  dInter_ = nullptr;
+  interRows_ = 0;
+  interUsed_ = false;
+  if (interDone_) (void)hipEventDestroy(interDone_);
+  interDone_ = nullptr;
   if (module_) (void)hipModuleUnload(module_);
   module_ = nullptr;
   function_ = nullptr;
+  for (Task& t : tasks_) t.function = nullptr;
   deviceReady_ = false;
 }
 
@@ -614,7 +695,43 @@ void Kernel::launch(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
   if (reinterpret_cast<uintptr_t>(dIn) % inputAlign_ != 0)
     fatal("RUNTIME ERROR: input pointer must be aligned to " + std::to_string(inputAlign_) + " bytes");
   if (reinterpret_cast<uintptr_t>(dOut) % bytesPerResult_ != 0) fatal("RUNTIME ERROR: output pointer is misaligned");
-  if (kind_ == SPNC_HIP_KERNEL_JIT) {
+  if (kind_ == SPNC_HIP_KERNEL_JIT && !tasks_.empty()) {
+    // The tasks one after the other on the caller's stream, over as many rows at a time as the intermediate buffer
+    // ("hip-task-buffer-mib", 1 GiB unless asked otherwise) holds: a multiple of 1024 rows, which keeps every chunk's input as aligned as the first.
+    const size_t rowBytes = size_t(numFeatures_) * bytesPerFeature_;
+    size_t chunk = n;
+    if (taskSlots_) {
+      const size_t most = std::max<size_t>(1024, (size_t(taskBufferMiB_) << 20) / (size_t(taskSlots_) * bytesPerResult_) / 1024 * 1024);
+      chunk = std::min(n, most);
+      if (interUsed_) hipCheck(hipStreamWaitEvent(stream, interDone_, 0), "hipStreamWaitEvent");
+      if (chunk > interRows_) {
+        if (dInter_) hipCheck(hipFree(dInter_), "hipFree(intermediate values)");  // waits for the device to finish with it
+        dInter_ = nullptr;
+        interRows_ = 0;
+        hipCheck(hipMalloc(&dInter_, size_t(taskSlots_) * chunk * bytesPerResult_), "hipMalloc(intermediate values)");
+        interRows_ = chunk;
+      }
+    }
+    for (size_t off = 0; off < n; off += chunk) {
+      const size_t rows = std::min(chunk, n - off);
+      const void* in = static_cast<const char*>(dIn) + off * rowBytes;
+      void* out = static_cast<char*>(dOut) + off * bytesPerResult_;
+      unsigned long long n64 = rows;
+      for (const Task& t : tasks_) {
+        const size_t tiles = (rows + t.blockSize - 1) / t.blockSize;
+        size_t cap = size_t(numCUs_) * t.blocksPerCU;
+        if (t.gridPolicy < 0) cap = tiles;
+        else if (t.gridPolicy > 0) cap = size_t(numCUs_) * t.gridPolicy;
+        const unsigned grid = unsigned(std::min<size_t>(std::min<size_t>(tiles, cap), 0x7fffffffu));
+        void* args[] = {(void*)&in, (void*)&out, (void*)&n64, (void*)&dInter_, (void*)&dInter_};
+        hipCheck(hipModuleLaunchKernel(t.function, grid, 1, 1, t.blockSize, 1, 1, 0, stream, args, nullptr), "kernel launch");
+      }
+    }
+    if (taskSlots_) {
+      hipCheck(hipEventRecord(interDone_, stream), "hipEventRecord");
+      interUsed_ = true;
+    }
+  } else if (kind_ == SPNC_HIP_KERNEL_JIT) {
     const size_t tile = size_t(blockSize_) * samplesPerLane_;
     const size_t tiles = (n + tile - 1) / tile;
     size_t cap = size_t(numCUs_) * blocksPerCU_;

@@ -68,6 +68,18 @@ class Kernel {
   std::string entry_;
   unsigned blockSize_ = 256, samplesPerLane_ = 1, inputAlign_ = 4;
   int gridPolicy_ = 0;  // 0 = resident blocks, -1 = one tile per block, n = n blocks per CU
+  // A graph cut by "maxTaskSize": several kernels in the one code object, launched one after the other on the caller's
+  // stream; values pass from task to task through an intermediate buffer of `taskSlots_` rows.
+  struct Task {
+    std::string entry;
+    unsigned blockSize = 256;
+    int gridPolicy = 0;
+    hipFunction_t function = nullptr;
+    int blocksPerCU = 1;
+  };
+  std::vector<Task> tasks_;
+  unsigned taskSlots_ = 0;
+  unsigned taskBufferMiB_ = 1024;
   // interpreter
   InterpProgram prog_;
 
@@ -100,6 +112,12 @@ class Kernel {
   } stage_[2];
   size_t stageRows_ = 0;
   hipEvent_t kernelDone_ = nullptr;
+  // intermediate buffer of a partitioned kernel: [taskSlots_][interRows_] results, reused by every call (calls on
+  // different streams wait for each other through interDone_)
+  void* dInter_ = nullptr;
+  size_t interRows_ = 0;
+  hipEvent_t interDone_ = nullptr;
+  bool interUsed_ = false;
 };
 
 }  // namespace spnc_hip

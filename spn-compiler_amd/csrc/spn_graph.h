@@ -11,7 +11,9 @@
 
 namespace spnc_hip {
 
-enum class NodeKind : uint8_t { Product = 0, Sum = 1, Histogram = 2, Gaussian = 3, Categorical = 4 };
+// External: inside one task of a partitioned graph, the value of a node that an earlier task computed (`feature` is its
+// row in the intermediate buffer). Never appears in the graph of a whole query.
+enum class NodeKind : uint8_t { Product = 0, Sum = 1, Histogram = 2, Gaussian = 3, Categorical = 4, External = 5 };
 
 // A node exactly as serialized (ids, scope values).
 struct RawNode {
@@ -119,7 +121,26 @@ struct Graph {
   // because every path from the root meets a leaf of that feature (what the kernels may rely on for such inputs).
   bool completeDecomposable = false;
   uint32_t root() const { return uint32_t(nodes.size() - 1); }
+  // One task of a graph cut by "maxTaskSize": the values of `taskOutputs` go to rows `taskOutputSlots` of the intermediate
+  // buffer ([rows][samples], value-major, so that the lanes of a wavefront touch consecutive addresses); the task that
+  // holds the whole graph's root (`taskFinal`; the root is its last node) writes the result instead.
+  bool isTask = false, taskFinal = false;
+  std::vector<uint32_t> taskOutputs, taskOutputSlots;
 };
+
+// A graph cut into tasks that run one after the other, each a kernel of its own (the reference's
+// mlir/lib/Dialect/LoSPN/Passes/LoSPNTaskPartitioner.cpp:36-148). `slots` rows of intermediate values are live at most.
+struct TaskPlan {
+  std::vector<Graph> tasks;
+  uint32_t slots = 0;
+};
+// Operations of a node as the reference's partitioner counts them on the binarised graph: one per leaf, k-1 multiplies
+// per k-ary product, k multiplies by the weights and k-1 adds per k-ary sum.
+uint64_t taskWeight(const GraphNode& n);
+uint64_t taskWeight(const Graph& g);
+// Cuts `g` into tasks of at most `maxTaskSize` operations (plus 1 % slack, at least one). Sums and products that alone
+// exceed the bound are first split into trees of smaller ones. One task (the graph itself, unmarked) if it fits.
+TaskPlan partitionGraph(const Graph& g, int maxTaskSize);
 
 // Validates the query and builds the scheduled DAG: only nodes reachable from the root,
 // depth-first post-order (children first, left to right), structurally identical nodes merged.

@@ -45,6 +45,8 @@ class _Info(ctypes.Structure):
         ("fused_min", ctypes.c_uint64),
         ("feature_is_float", ctypes.c_uint),
         ("support_marginal", ctypes.c_uint),
+        ("num_tasks", ctypes.c_uint),
+        ("task_rows", ctypes.c_uint),
     ]
 
 

@@ -101,12 +101,12 @@ def test_option_handling(native):
     os.remove(k.fileName())
     with pytest.raises(RuntimeError, match="Could not parse option value"):
         compile_query(native, path, **{"hip-kernel": "magic"})
-    # maxTaskSize: a graph above the bound runs on the interpreter instead of being cut into tasks
+    # maxTaskSize: a graph above the bound is cut into tasks, one kernel each
     k = compile_query(native, path, maxTaskSize=10)
-    assert k.info()["kernel_kind"] == 2
+    assert k.info()["kernel_kind"] == 1 and k.info()["num_tasks"] > 1 and k.info()["task_rows"] >= 1
     os.remove(k.fileName())
     k = compile_query(native, path, maxTaskSize=100000)
-    assert k.info()["kernel_kind"] == 1
+    assert k.info()["kernel_kind"] == 1 and k.info()["num_tasks"] == 1 and k.info()["task_rows"] == 0
     os.remove(k.fileName())
     with pytest.raises(RuntimeError, match="hip-interp-staged-features must be lds, spill or auto"):
         compile_query(native, path, **{"hip-kernel": "interpreter", "hip-interp-staged-features": "hbm"})
@@ -411,3 +411,34 @@ def test_kernel_file_round_trip(native):
         native.Kernel("/nonexistent/kernel.hipk")
     with pytest.raises(RuntimeError, match="not a spnc-hip kernel file"):
         native.Kernel(os.path.join(GOLDEN, "NIPS5.bin"))
+
+
+@pytest.mark.parametrize("name,size", [("NIPS5", 3), ("NIPS5", 10), ("nltcs", 100), ("plants", 5), ("plants", 700)])
+def test_max_task_size_cuts_the_graph_into_bounded_tasks(native, tmp_path, name, size):
+    """maxTaskSize as in the reference (mlir/lib/Dialect/LoSPN/Partitioning/GraphPartitioner.cpp:84-157): tasks of at
+    most that many operations plus 1 % slack (at least one), each a kernel of its own in one code object; every value
+    a task hands on has a row of the intermediate buffer, and only the last task writes the result."""
+    import re
+    if name == "NIPS5":
+        path = os.path.join(GOLDEN, "NIPS5.bin")
+    else:
+        path = model_as_query(os.path.join(GOLDEN, name + ".bin"), "float64", str(tmp_path / "q.bin"))
+    k = compile_query(native, path, maxTaskSize=size, **{"hip-kernel": "jit"})
+    src, info = k.source(), k.info()
+    heads = re.findall(r"// task (\d+) of (\d+): (\d+) operations, (\d+) values in, (\d+) values out(, the result)?", src)
+    assert len(heads) == info["num_tasks"] > 1
+    slack = max(1, int(size * 0.01))
+    # a binary sum is three operations (two weights, one add) and cannot be cut further
+    assert all(int(h[2]) <= max(size + slack, 3) for h in heads)
+    assert [h[5] != "" for h in heads] == [False] * (len(heads) - 1) + [True]
+    assert int(heads[0][3]) == 0 and int(heads[-1][4]) == 0
+    assert sum(int(h[4]) for h in heads) >= len(heads) - 1
+    for t in range(len(heads)):
+        assert 'void __launch_bounds__(SPN_BLOCK) spn_task%d(' % t in src or 'spn_task%d(' % t in src
+    rows = [int(r) for r in re.findall(r"spn_res\[(\d+)ull \* spn_n\]", src)] + [int(r) for r in re.findall(r"spn_in\[(\d+)ull \* spn_n\]", src)]
+    assert max(rows) + 1 == info["task_rows"]
+    # the kernel file keeps the tasks
+    k2 = native.Kernel(k.fileName(), k.kernelName(), k.queryType(), k.target(), k.batchSize(), k.numFeatures(), k.bytesPerFeature(), k.numResults(),
+                       k.bytesPerResult(), k.dataType())
+    assert k2.info()["num_tasks"] == info["num_tasks"] and k2.info()["task_rows"] == info["task_rows"]
+    os.remove(k.fileName())
