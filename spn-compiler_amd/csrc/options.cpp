@@ -94,6 +94,8 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       if (o.samplesPerLane < 0 || o.samplesPerLane > 16) throw std::runtime_error("hip-samples-per-lane must be in [0,16]");
     } else if (key == "hip-jit-max-ops") {
       o.jitMaxOps = parseInt(key, val);
+    } else if (key == "hip-nan-masks") {
+      o.nanMasks = parseBool(val);
     } else if (key == "hip-task-buffer-mib") {
       o.taskBufferMiB = parseInt(key, val);
       if (o.taskBufferMiB < 1 || o.taskBufferMiB > 65536) throw std::runtime_error("hip-task-buffer-mib must be in [1,65536]");

@@ -54,6 +54,7 @@ struct CompileOptions {
   long interpLongRange = -1;                   // "hip-interp-long-range": values living longer than this many instructions go to the long-lived pool (-1 = automatic)
   int packedRows = -1;                         // "hip-packed-rows": wide rows of small integer features stay packed four to a register and the table leaves of sibling products are evaluated together (1), not (0), decided per kernel (-1)
   int oneHotMaxDomain = 3;                     // "hip-one-hot-max-domain": with packed rows, table leaves over at most this many categories are evaluated as multiply-adds on the vector unit instead of LDS reads
+  bool nanMasks = true;                        // "hip-nan-masks": with marginalisation in log space, a Gaussian leaf of a missing (NaN) feature is zeroed by a bitwise AND with a per-feature mask instead of a select per leaf
   int taskBufferMiB = 1024;                    // "hip-task-buffer-mib": most device memory the values passing between the tasks of a partitioned graph may take; larger batches run in several passes
   int prefetchRows = -1;                       // "hip-prefetch-rows": with the per-wavefront transposed load, the loads of a wavefront's next 64 rows are issued before the current ones are evaluated and stay in registers meanwhile (-1 = with packed rows)
   bool hoistFeatureValues = true;              // "hip-hoist-feature-values": with packed rows, the values (and squares) of the features whose leaves are polynomials are computed once at the top of the kernel (false = again in every group of products that uses them: more arithmetic, fewer registers)
