@@ -66,12 +66,15 @@ def main():
     # ---- calibration: what the traffic counters read for a copy of known size ----
     units, copy_lines = {}, []
     for counter in ("FETCH_SIZE", "WRITE_SIZE"):
-        con, _, shown = rocprof(work, "copy_" + counter, ["--pmc", counter], ["--copy-gib", "4", "--steps", "5"])
-        value = max(r[1] for r in counters(con, "%"))
+        con, _, shown = rocprof(work, "copy_" + counter, ["--pmc", counter], ["--copy-gib", "4", "--steps", "5", "--warmup", "1"])
+        # all dispatches of the copy kernel (the library may split one copy over several), not the fill that makes its input
+        total = con.execute("select sum(counter_value) from pmc_events where counter_name = ? and (name like '%Mul%' or name like '%mul%')",
+                            (counter,)).fetchone()[0]
+        value = total / 6.0   # per copy: five timed and one warm-up
         units[counter] = 4 * 1048576.0 / value      # KiB per counter unit
-        copy_lines += ["$ " + shown, "%-46s %-12s per-dispatch=%.1f" % ("copy kernel", counter, value)]
+        copy_lines += ["$ " + shown, "%-46s %-12s per 4 GiB copy=%.1f" % ("copy kernel", counter, value)]
     with open(os.path.join(prof, "copy_kernel_counters.txt"), "w") as f:
-        f.write("Plain device-to-device copy of 4 GiB (torch Tensor.copy_), the reference point for the FETCH_SIZE and WRITE_SIZE\n"
+        f.write("Plain copy kernel over 4 GiB (torch.mul(a, 1.0, out=b) on float32), the reference point for the FETCH_SIZE and WRITE_SIZE\n"
                 "counters of rocprofv3 on MI355X: the copy reads 4 GiB and writes 4 GiB (4194304 KiB each; far more than the 256 MiB\n"
                 "of last-level cache could hold back from HBM).\n"
                 "Made by: python3 profile_counters.py\n\n" + "\n".join(copy_lines) +

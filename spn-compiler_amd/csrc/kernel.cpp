@@ -277,7 +277,12 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
   } else {
     k->kind_ = SPNC_HIP_KERNEL_JIT;
     TaskPlan plan;
-    if (o.maxTaskSize > 0) plan = partitionGraph(g, o.maxTaskSize);
+    // Without "maxTaskSize", a graph that is larger than what one straight-line kernel is built for (it is here because
+    // linear-space computation or the caller ruled the interpreter out) is cut into tasks of 2000 operations: hipRTC
+    // time then grows with the graph instead of with its square, and no kernel outgrows the register file.
+    int taskSize = o.maxTaskSize;
+    if (taskSize <= 0 && ops > jitLimit && o.kernelMode != KernelMode::Jit) taskSize = 2000;
+    if (taskSize > 0) plan = partitionGraph(g, taskSize);
     JitSource js;
     if (plan.tasks.size() > 1) {
       // One translation unit with a kernel per task: each task's source in a namespace of its own, the macros it

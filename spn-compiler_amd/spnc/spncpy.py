@@ -54,6 +54,29 @@ def library_path():
     return os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), _LIB_NAME)
 
 
+def _share_torch_hip_runtime():
+    """One process, one HIP runtime. PyTorch ships a copy of libamdhip64 and asks the loader for it by a name that an
+    already loaded system copy does not answer to; loaded second, that copy finds no GPU ("No HIP GPUs are
+    available"). The other way round works: this library asks for the runtime by its soname, which PyTorch's copy
+    carries too. So where PyTorch is installed but not imported yet, its copy is loaded first, by path."""
+    import importlib.util
+    import sys
+    if "torch" in sys.modules:
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    if spec is None or not spec.submodule_search_locations:
+        return
+    runtime = os.path.join(list(spec.submodule_search_locations)[0], "lib", "libamdhip64.so")
+    if os.path.isfile(runtime):
+        try:
+            ctypes.CDLL(runtime, mode=ctypes.RTLD_GLOBAL)
+        except OSError:
+            pass  # not loadable on its own: the system's runtime serves this library
+
+
 def _load():
     global _lib
     if _lib is not None:
@@ -61,6 +84,7 @@ def _load():
     path = library_path()
     if not os.path.isfile(path):
         raise RuntimeError(f"{_LIB_NAME} not found at {path}; build it with `make -C spn-compiler_amd/csrc`")
+    _share_torch_hip_runtime()
     lib = ctypes.CDLL(path)
     vp, cp, sz = ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t
     lib.spnc_hip_available.restype = ctypes.c_int

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 import rawfile as rf
-from conftest import GOLDEN, compile_query, compile_spn, load_golden, model_as_query, oracle_model, quiet
+from conftest import GOLDEN, ROOT, compile_query, compile_spn, load_golden, model_as_query, oracle_model, quiet
 from oracle import c_oracle, evaluate as ev, spn_model as sm
 
 pytestmark = pytest.mark.gpu
@@ -119,7 +119,7 @@ def test_golden_outputs_f32(native, tmp_path, name, variant):
                          ids=["log-f64", "log-f64-pairwise", "log-f64-interp", "linear-f64"])
 @pytest.mark.parametrize("name", ["NIPS5", "nltcs", "plants"])
 def test_golden_outputs_f64(native, tmp_path, name, opts):
-    if name == "nltcs" and ("hip-sum-form" in opts or "use-log-space" in opts):
+    if name == "nltcs" and "hip-sum-form" in opts:
         # one straight-line float64 kernel of the 3641-node model takes minutes of hipRTC time: cut into tasks it builds in seconds
         opts = dict(opts, maxTaskSize=300, **{"hip-kernel": "jit"})
     X, ref = load_golden(name)
@@ -127,7 +127,11 @@ def test_golden_outputs_f64(native, tmp_path, name, opts):
         path, X = os.path.join(GOLDEN, "NIPS5.bin"), X.astype(np.uint32)
     else:
         path = model_as_query(os.path.join(GOLDEN, name + ".bin"), "float64", str(tmp_path / "q.bin"))
-    got = run(compile_query(native, path, **opts), X)
+    k = compile_query(native, path, **opts)
+    if name == "nltcs" and "use-log-space" in opts:
+        # linear space rules the interpreter out; a graph this size is cut into tasks without being asked
+        assert k.info()["kernel_kind"] == 1 and k.info()["num_tasks"] > 1
+    got = run(k, X)
     assert got.dtype == np.float64
     assert np.abs(got - ref).max() <= F64_TOL
 
@@ -758,3 +762,41 @@ def test_quads_of_leaf_regions_inside_the_outer_sum(native, count, leaves, regio
         got = run(k, X)
         assert got.dtype == np.float32
         assert np.abs(got - want64).max() <= F32_TOL * max(1.0, np.abs(want64).max() / 100), opts
+
+
+_LOAD_ORDER_SCRIPT = r"""
+import os, sys
+import numpy as np
+root = sys.argv[1]
+sys.path.insert(0, os.path.join(root, "spn-compiler_amd")); sys.path.insert(0, os.path.join(root, "tests")); sys.path.insert(0, root)
+from spnc import spncpy as native
+from spnc.hip import HIPCompiler
+from spnc.structure import Categorical, Product
+assert "torch" not in sys.modules
+p = Product(children=[Categorical(p=[.35, .55, .1], scope=0), Categorical(p=[.25, .625, .125], scope=1)])
+X = np.array([[0, 1], [2, 2], [1, 0]], dtype=np.int32)
+k = HIPCompiler().compile_ll(p, "int32", supportMarginal=False)
+first = k.execute(3, X)                       # the library's HIP runtime is up before torch is even imported
+import torch
+t = torch.arange(1000, device="cuda", dtype=torch.float32)
+assert float(t.sum()) == 499500.0
+second = k.execute(3, X)
+Xd = torch.from_numpy(X).cuda()
+out = torch.empty(3, dtype=torch.float32, device="cuda")
+torch.cuda.synchronize()
+k.execute_device(3, Xd.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+torch.cuda.synchronize()
+want = np.log(np.array([.35 * .625, .1 * .125, .55 * .25]))
+for got in (first, second, out.cpu().numpy()):
+    assert np.abs(got - want).max() < 1e-6, got
+os.remove(k.fileName())
+print("load order ok")
+"""
+
+
+def test_library_loaded_before_torch(native):
+    """The library brought up first, PyTorch imported and used afterwards, in a fresh process: both must work on the one
+    GPU whichever HIP runtime library the loader picked for the process."""
+    import subprocess, sys
+    r = subprocess.run([sys.executable, "-c", _LOAD_ORDER_SCRIPT, ROOT], capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0 and "load order ok" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
