@@ -27,7 +27,7 @@ sys.path.insert(0, os.path.join(ROOT, "spn-compiler_amd"))
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X FP32 vector, published
 FP64_VECTOR_PEAK_TFLOPS = 78.6   # MI355X FP64 vector, published
-ALL = ["c1", "c2", "c3", "c4", "c5", "c5_f64"]
+ALL = ["c1", "c2", "c3", "c4", "c5", "c5_f64", "c4_f64"]
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
 
@@ -83,8 +83,8 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None, fast_inpu
     from spnc import synthetic as syn
     from spnc.hip import HIPCompiler
     workload_key, extra_given = name, bool(extra_options)
-    if name == "c5_f64":   # configuration 5 computed in float64 log-space
-        name, extra_options = "c5", dict(extra_options or {}, **{"hip-compute-type": "float64"})
+    if name.endswith("_f64"):   # the same configuration computed in float64 log-space (c5: straight-line kernel, c4: interpreter)
+        name, extra_options = name[:-4], dict(extra_options or {}, **{"hip-compute-type": "float64"})
     cfg = syn.CONFIGS[name]
     n = n or cfg["n"]
     spn = cfg["spn"]()
@@ -270,7 +270,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="c1", choices=["c1", "c2", "c3", "c3_deep", "c4", "c5", "c5_f64"])
+    ap.add_argument("--config", default="c1", choices=["c1", "c2", "c3", "c3_deep", "c4", "c5", "c5_f64", "c4_f64"])
     ap.add_argument("--n", type=int, default=0, help="override the number of samples")
     ap.add_argument("--no-others", action="store_true", help="measure only the selected configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
@@ -348,7 +348,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f64" if args.config == "c5_f64" else "f32",
+        "dtype": "f64" if args.config.endswith("_f64") else "f32",
         "data": ("synthetic (seeded NumPy generators for SPN parameters; inputs drawn on the device)" if args.fast_inputs else
                  "synthetic (seeded NumPy generators for SPN parameters and inputs, the arrays of the parity tests; inputs resident in HBM "
                  "before the timed region)"),

@@ -8,7 +8,7 @@ FETCH_SIZE and WRITE_SIZE, then two sets of SQ counters), each in a pass of its 
   profiles/copy_kernel_counters.txt  what the traffic counters read for a plain 4 GiB device copy (their calibration)
   profiles/traffic.json            HBM bytes per launch per configuration, with bench.py's key of the kernel measured
 
-usage: python3 profile_counters.py [config ...]       (default: all six; raw profiler output goes to a temporary directory)
+usage: python3 profile_counters.py [config ...]       (default: all seven; raw profiler output goes to a temporary directory)
 """
 import glob
 import json
@@ -22,7 +22,7 @@ import tempfile
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 BENCH = os.path.join(ROOT, "bench.py")
-KERNELS = {"c1": "spn_kernel", "c2": "spn_kernel", "c3": "spn_kernel", "c4": "spn_interp_kernel", "c5": "spn_kernel", "c5_f64": "spn_kernel"}
+KERNELS = {"c1": "spn_kernel", "c2": "spn_kernel", "c3": "spn_kernel", "c4": "spn_interp_kernel", "c5": "spn_kernel", "c5_f64": "spn_kernel", "c4_f64": "spn_interp_kernel"}
 SQ_SETS = [
     "SQ_INSTS_VALU SQ_INSTS_SALU SQ_INSTS_SMEM SQ_INSTS_LDS SQ_WAVE_CYCLES SQ_BUSY_CYCLES SQ_ACTIVE_INST_VALU SQ_WAIT_INST_ANY",
     "SQ_WAVES SQ_INSTS_VALU_TRANS SQ_ACTIVE_INST_LDS SQ_LDS_BANK_CONFLICT SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR SQ_INSTS_MFMA SQ_ACTIVE_INST_ANY",

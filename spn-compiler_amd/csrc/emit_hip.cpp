@@ -1032,6 +1032,21 @@ unsigned pickVectorBytes(unsigned rowBytes, unsigned elemBytes) {
 
 }  // namespace
 
+std::vector<double> doubleMathTables() {
+  std::vector<double> t;
+  for (int j = 0; j < 64; ++j) t.push_back(double(exp2l((long double)j / 64.0L)));
+  for (int j = 0; j < 256; ++j) {
+    const double recip = double(1.0L / (1.0L + (long double)j / 256.0L));
+    t.push_back(recip);
+    t.push_back(j == 0 ? 0.0 : double(-log2l((long double)recip)));
+  }
+  static const double poly[12] = {0x1.5d87fe78a6731p-10, 0x1.3b2ab6fba4e77p-7, 0x1.c6b08d704a0cp-5, 0x1.ebfbdff82c58fp-3, 0x1.62e42fefa39efp-1,
+                                  0x1.a61762a7aded9p-3, -0x1.ec709dc3a03fdp-3, 0x1.2776c50ef9bfep-2, -0x1.71547652b82fep-2,
+                                  0x1.ec709dc3a03fdp-2, -0x1.71547652b82fep-1, 0x1.71547652b82fep+0};
+  t.insert(t.end(), poly, poly + 12);
+  return t;
+}
+
 JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::string& entry) {
   Emitter e(g, o);
   // Short rows are fetched with the widest vector loads their size allows, all samples of a
@@ -1179,21 +1194,18 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
     // (remainder 2e-18 relative). Both agree with the library to 1e-15 relative over their ranges (checked on
     // the CPU against exp2/log2 of libm). The tables live in LDS, 4.5 KiB per block.
     s << "#define SPN_DOUBLE_TABLES 1\n";
+    const std::vector<double> math = doubleMathTables();
     s << "__device__ const real_t spn_exp2_table[64] = {";
-    for (int j = 0; j < 64; ++j) s << (j ? ", " : "") << (j % 4 == 0 ? "\n  " : "") << e.lit(double(exp2l((long double)j / 64.0L)));
+    for (int j = 0; j < 64; ++j) s << (j ? ", " : "") << (j % 4 == 0 ? "\n  " : "") << e.lit(math[j]);
     s << "};\n__device__ const real_t spn_log2_table[512] = {";
-    for (int j = 0; j < 256; ++j) {
-      const double recip = double(1.0L / (1.0L + (long double)j / 256.0L));
-      const double lg = j == 0 ? 0.0 : double(-log2l((long double)recip));
-      s << (j ? ", " : "") << (j % 2 == 0 ? "\n  " : "") << e.lit(recip) << ", " << e.lit(lg);
-    }
+    for (int j = 0; j < 512; ++j) s << (j ? ", " : "") << (j % 4 == 0 ? "\n  " : "") << e.lit(math[64 + j]);
     s << "};\n";
     // The polynomial coefficients are read from LDS as well, once per kernel, and stay in registers: as literals
     // every use costs two register moves, since a double constant cannot be an operand of the instruction itself.
     // c5..c1 of exp2, then l7..l1 of log2.
-    s << "__device__ const real_t spn_poly[12] = {0x1.5d87fe78a6731p-10, 0x1.3b2ab6fba4e77p-7, 0x1.c6b08d704a0cp-5, 0x1.ebfbdff82c58fp-3, "
-         "0x1.62e42fefa39efp-1,\n  0x1.a61762a7aded9p-3, -0x1.ec709dc3a03fdp-3, 0x1.2776c50ef9bfep-2, -0x1.71547652b82fep-2, "
-         "0x1.ec709dc3a03fdp-2, -0x1.71547652b82fep-1, 0x1.71547652b82fep+0};\n";
+    s << "__device__ const real_t spn_poly[12] = {";
+    for (int j = 0; j < 12; ++j) s << (j ? ", " : "") << e.lit(math[576 + j]);
+    s << "};\n";
     s << "#ifndef SPN_EXP2_TABLE\n__shared__ real_t spn_exp2_lds[64];\n__shared__ __attribute__((aligned(16))) real_t spn_log2_lds[512];\n"
          "__shared__ real_t spn_poly_lds[12];\n"
          "#define SPN_EXP2_TABLE spn_exp2_lds\n#define SPN_LOG2_TABLE spn_log2_lds\n#define SPN_POLY spn_poly_lds\n#endif\n";

@@ -24,6 +24,7 @@ struct InterpLaunch {
   uint32_t ldsSlots;         // slots [0, ldsSlots) live in LDS, the rest in the spill tier
   uint32_t spillSlots;       // number of slots in the spill tier
   uint32_t marginal;         // NaN features marginalise Gaussian leaves
+  uint32_t mathTables;       // float64 in the log2 domain: index into `tables` of the exp2/log2 routines' tables
 };
 
 // Enqueues the interpreter on `stream`. ldsBytes = ldsSlots * INTERP_BLOCK * sizeof(compute type).

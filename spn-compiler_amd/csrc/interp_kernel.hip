@@ -17,13 +17,14 @@ const void* interpKernel_f32_natural_direct(int mode);
 const void* interpKernel_f32_natural_staged(int mode);
 const void* interpKernel_f32_natural_registers(int mode);
 const void* interpKernel_f64(int mode);
+const void* interpKernel_f64_log2(int mode);
 
 namespace {
 
 // float kernels exist once per feature mode: the fused leaf instructions are long, and a kernel that held both
 // of their forms would run the staged one slower (instruction fetch). double kernels decide at run time.
 const void* pick(bool f64, bool log2Domain, int mode, uint32_t featureMode) {
-  if (f64) return interpKernel_f64(mode);
+  if (f64) return log2Domain ? interpKernel_f64_log2(mode) : interpKernel_f64(mode);
   if (featureMode == FEAT_REGISTER) return log2Domain ? interpKernel_f32_log2_registers(mode) : interpKernel_f32_natural_registers(mode);
   if (featureMode == FEAT_STAGED) return log2Domain ? interpKernel_f32_log2_staged(mode) : interpKernel_f32_natural_staged(mode);
   return log2Domain ? interpKernel_f32_log2_direct(mode) : interpKernel_f32_natural_direct(mode);

@@ -54,6 +54,50 @@ struct Math<double, false> {
   static __device__ __forceinline__ double lowest() { return -1.7976931348623157e308; }
 };
 
+// float64 in the log2 domain: base-2 exponential and logarithm by table and short polynomial, the routines that
+// the straight-line float64 kernels carry (emit_hip.cpp): 2^x = 2^(n>>6) * T[n&63] * 2^r with n = rint(64 x),
+// |r| <= 1/128 and a degree-5 polynomial; log2(2^e t) = e + G[j] + log2(1 + u), j = the top eight fraction bits of t,
+// u = t R[j] - 1 in one fma, degree-7 polynomial. Within 1e-15 of libm. The tables (doubleMathTables()) are copied from
+// behind the program's leaf tables into LDS when the kernel starts.
+__shared__ double mathExp2[64];
+__shared__ __align__(16) double mathLog2[512];
+__shared__ double mathPoly[12];
+template <>
+struct Math<double, true> {
+  static __device__ __forceinline__ double exp(double x) {
+    x = x < -1100.0 ? -1100.0 : x;  // keeps NaN
+    const double n = __builtin_rint(x * 64.0), r = __builtin_fma(n, -0x1p-6, x);
+    const int ni = (int)n;
+    const double t = mathExp2[ni & 63];
+    double p = mathPoly[0];
+    p = __builtin_fma(p, r, mathPoly[1]);
+    p = __builtin_fma(p, r, mathPoly[2]);
+    p = __builtin_fma(p, r, mathPoly[3]);
+    p = __builtin_fma(p, r, mathPoly[4]);
+    return __builtin_ldexp(__builtin_fma(t, p * r, t), ni >> 6);
+  }
+  static __device__ __forceinline__ double log(double x) {
+    union { double d; unsigned long long u; } c;
+    c.d = x;
+    const unsigned hi = (unsigned)(c.u >> 32);
+    const int e = (int)(hi >> 20) - 1023;
+    const unsigned j = (hi >> 12) & 255u;
+    c.u = (c.u & 0x000fffffffffffffull) | 0x3ff0000000000000ull;
+    const double u = __builtin_fma(c.d, mathLog2[2 * j], -1.0);
+    double p = mathPoly[5];
+    p = __builtin_fma(p, u, mathPoly[6]);
+    p = __builtin_fma(p, u, mathPoly[7]);
+    p = __builtin_fma(p, u, mathPoly[8]);
+    p = __builtin_fma(p, u, mathPoly[9]);
+    p = __builtin_fma(p, u, mathPoly[10]);
+    p = __builtin_fma(p, u, mathPoly[11]);
+    const double r = __builtin_fma(u, p, mathLog2[2 * j + 1] + (double)e);
+    return x == 0.0 ? -__builtin_huge_val() : (x != x ? x : r);  // 0: a sum whose terms are all impossible
+  }
+  static __device__ __forceinline__ double finish(double x) { return x * 0x1.62e42fefa39efp-1; }
+  static __device__ __forceinline__ double lowest() { return -1.7976931348623157e308; }
+};
+
 __device__ __forceinline__ float rmax(float a, float b) { return __builtin_fmaxf(a, b); }
 __device__ __forceinline__ double rmax(double a, double b) { return __builtin_fmax(a, b); }
 __device__ __forceinline__ float rfma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
@@ -979,6 +1023,13 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
   Sl.spill = Sg.spill;
   Sl.spillBlock = Sg.spillBlock;
   Sl.ldsSlots = Sg.ldsSlots;
+  if (sizeof(R) == 8 && LOG2) {
+    const double* math = static_cast<const double*>(a.tables) + a.mathTables;
+    for (unsigned t = threadIdx.x; t < 64; t += B) mathExp2[t] = math[t];
+    for (unsigned t = threadIdx.x; t < 512; t += B) mathLog2[t] = math[64 + t];
+    if (threadIdx.x < 12) mathPoly[threadIdx.x] = math[576 + threadIdx.x];
+    __syncthreads();
+  }
   const unsigned long long F = a.numFeatures;
   const bool stagedMode = FEAT == 2 ? a.featureMode == FEAT_STAGED : FEAT == 1;
   FeatureRegs regs;

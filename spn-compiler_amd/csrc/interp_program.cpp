@@ -1,5 +1,7 @@
 #include "interp_program.h"
 
+#include "emit_hip.h"
+
 #include <algorithm>
 #include <cmath>
 #include <cstring>
@@ -95,8 +97,17 @@ InterpProgram buildInterpProgram(const Graph& g, const CompileOptions& o) {
         best = std::move(p);
         have = true;
       }
-      if (best.spillAccesses == 0 && rank(best) == 0) return best;
+      if (best.spillAccesses == 0 && rank(best) == 0) break;
     }
+    if (have && best.spillAccesses == 0 && rank(best) == 0) break;
+  }
+  if (best.f64 && best.log2Domain) {
+    // The tables of the float64 exp2/log2 routines travel behind the leaf tables (16-byte aligned: the kernel copies
+    // them into LDS when it starts).
+    if (best.tables.size() % 2) best.tables.push_back(0.0);
+    best.mathTables = uint32_t(best.tables.size());
+    const std::vector<double> math = doubleMathTables();
+    best.tables.insert(best.tables.end(), math.begin(), math.end());
   }
   return best;
 }
@@ -114,7 +125,8 @@ void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures) {
   if (p.featureMode != FEAT_STAGED && p.featureMode != FEAT_DIRECT && p.featureMode != FEAT_REGISTER) bad("feature mode", 0);
   const bool inRegisters = p.featureMode == FEAT_REGISTER;
   if (inRegisters && (p.f64 || p.staged.size() > 32)) bad("register features", 0);
-  if (p.f64 && p.log2Domain) bad("compute type", 0);
+  if ((p.f64 && p.log2Domain) != (p.mathTables != 0xFFFFFFFFu)) bad("math tables", 0);
+  if (p.mathTables != 0xFFFFFFFFu && (p.mathTables % 2 != 0 || size_t(p.mathTables) + DOUBLE_MATH_TABLE_VALUES > p.tables.size())) bad("math tables", 0);
   std::map<uint32_t, uint32_t> indexBound;  // staged index slot -> largest index it can hold
   std::set<uint32_t> valueSlots;
   for (size_t k = 0; k < p.staged.size(); ++k) {
@@ -288,7 +300,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   if (!o.useLogSpace) throw std::runtime_error("The interpreter kernel supports log-space computation only");
   InterpProgram p;
   p.f64 = o.computeType == ComputeType::F64;
-  p.log2Domain = !p.f64 && o.log2Domain;
+  p.log2Domain = o.log2Domain;
   Builder b(g, p);
   const size_t N = g.nodes.size();
   auto isLeaf = [&](uint32_t i) { return g.nodes[i].kind != NodeKind::Product && g.nodes[i].kind != NodeKind::Sum; };

@@ -81,6 +81,7 @@ struct InterpProgram {
   uint32_t shortSlots = 0;    // slots [0, shortSlots) are the busy ones; [shortSlots, numSlots) hold long-lived values
   uint32_t reservedSlots = 0; // leading slots pinned to staged features
   uint32_t numInstructions = 0;
+  uint32_t mathTables = 0xFFFFFFFFu;  // float64 in the log2 domain: where in `tables` the 588 values of the exp2/log2 routines start
   uint32_t ldsSlotLimit = 0;  // "hip-interp-lds-slots": the launcher keeps at most this many slots in LDS (0 = as many as fit)
   uint32_t spillAccesses = 0; // slot words naming a long-lived slot: reads and writes of the spill tier per sample when only the short pool is in LDS
   std::string listing;        // human-readable form, for "dump-ir"

@@ -416,6 +416,7 @@ void Kernel::save(const std::string& path) const {
     w.u32(prog_.reservedSlots);
     w.u32(prog_.numInstructions);
     w.u32(prog_.ldsSlotLimit);
+    w.u32(prog_.mathTables);
   }
   FILE* f = std::fopen(path.c_str(), "wb");
   if (!f) fatal("COMPILATION ERROR: cannot write kernel file " + path);
@@ -483,6 +484,7 @@ std::unique_ptr<Kernel> Kernel::load(const std::string& kernelFile) {
     k->prog_.reservedSlots = r.u32();
     k->prog_.numInstructions = r.u32();
     k->prog_.ldsSlotLimit = r.u32();
+    k->prog_.mathTables = r.u32();
     k->inputAlign_ = k->bytesPerFeature_;
   } else {
     fatal("RUNTIME ERROR: unknown kernel kind in " + kernelFile);
@@ -770,6 +772,7 @@ void Kernel::launchProgram(size_t n, const void* dIn, void* dOut, const uint32_t
   a.ldsSlots = ldsSlots_;
   a.spillSlots = prog_.numSlots - ldsSlots_;
   a.marginal = marginal_ ? 1u : 0u;
+  a.mathTables = prog_.mathTables;
   hipCheck(launchInterpreter(a, prog_.f64, prog_.log2Domain, interpMode_, grid, ldsBytes_, stream), "interpreter launch");
 }
 

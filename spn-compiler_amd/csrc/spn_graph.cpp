@@ -166,6 +166,7 @@ std::string structuralKey(const GraphNode& g) {
   std::string key;
   key.push_back(char(g.kind));
   switch (g.kind) {
+    case NodeKind::External: break;  // only inside the tasks of a cut graph (partition.cpp), never here
     case NodeKind::Gaussian:
       appendBytes(key, &g.feature, 4);
       appendBytes(key, &g.mean, 8);
@@ -211,6 +212,7 @@ Graph buildGraph(const RawQuery& q) {
   for (size_t i = 0; i < m.nodes.size(); ++i) {
     const RawNode& n = m.nodes[i];
     switch (n.kind) {
+      case NodeKind::External: break;  // only inside the tasks of a cut graph (partition.cpp), never here
       case NodeKind::Product:
         if (n.children.empty()) fatal("Number of operands must be at least one");
         break;
@@ -257,6 +259,7 @@ Graph buildGraph(const RawQuery& q) {
     GraphNode gn;
     gn.kind = n.kind;
     switch (n.kind) {
+      case NodeKind::External: break;  // only inside the tasks of a cut graph (partition.cpp), never here
       case NodeKind::Product:
       case NodeKind::Sum:
         for (int32_t c : n.children) gn.children.push_back(placed.at(defined[c]));
@@ -333,6 +336,7 @@ Graph buildGraph(const RawQuery& q) {
     uint64_t k = n.children.size();
     st.maxFanIn = std::max<uint32_t>(st.maxFanIn, uint32_t(k));
     switch (n.kind) {
+      case NodeKind::External: break;  // only inside the tasks of a cut graph (partition.cpp), never here
       case NodeKind::Gaussian:
         st.gaussians++;
         st.flopsMin += 4 + leafSelect;
@@ -499,6 +503,7 @@ LoSpnStats computeLoSpnStats(const RawQuery& q, bool logSpace) {
     byId[n.id] = i;
     const uint64_t k = n.children.size();
     switch (n.kind) {
+      case NodeKind::External: break;  // only inside the tasks of a cut graph (partition.cpp), never here
       case NodeKind::Product: st.productCount += k ? k - 1 : 0; break;
       case NodeKind::Sum:
         st.sumCount += k ? k - 1 : 0;
