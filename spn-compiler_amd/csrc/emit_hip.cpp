@@ -1,5 +1,7 @@
 #include "emit_hip.h"
 
+#include "math_tables.h"
+
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
@@ -1031,21 +1033,6 @@ unsigned pickVectorBytes(unsigned rowBytes, unsigned elemBytes) {
 }
 
 }  // namespace
-
-std::vector<double> doubleMathTables() {
-  std::vector<double> t;
-  for (int j = 0; j < 64; ++j) t.push_back(double(exp2l((long double)j / 64.0L)));
-  for (int j = 0; j < 256; ++j) {
-    const double recip = double(1.0L / (1.0L + (long double)j / 256.0L));
-    t.push_back(recip);
-    t.push_back(j == 0 ? 0.0 : double(-log2l((long double)recip)));
-  }
-  static const double poly[12] = {0x1.5d87fe78a6731p-10, 0x1.3b2ab6fba4e77p-7, 0x1.c6b08d704a0cp-5, 0x1.ebfbdff82c58fp-3, 0x1.62e42fefa39efp-1,
-                                  0x1.a61762a7aded9p-3, -0x1.ec709dc3a03fdp-3, 0x1.2776c50ef9bfep-2, -0x1.71547652b82fep-2,
-                                  0x1.ec709dc3a03fdp-2, -0x1.71547652b82fep-1, 0x1.71547652b82fep+0};
-  t.insert(t.end(), poly, poly + 12);
-  return t;
-}
 
 JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::string& entry) {
   Emitter e(g, o);

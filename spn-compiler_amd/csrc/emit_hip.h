@@ -34,10 +34,4 @@ struct JitSource {
 // read from and to write to, [rows][n] values of the kernel's compute type.
 JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::string& entry = "spn_kernel");
 
-// Tables of the base-2 exponential and logarithm that float64 kernels carry with them (straight-line and interpreter):
-// 64 values 2^(j/64); 256 pairs (R[j], G[j]) = (1/(1+j/256) rounded, -log2 of that rounded value); the polynomial
-// coefficients c5..c1 of 2^r - 1 and l7..l1 of log2(1+u). 64 + 512 + 12 doubles.
-constexpr unsigned DOUBLE_MATH_TABLE_VALUES = 64 + 512 + 12;
-std::vector<double> doubleMathTables();
-
 }  // namespace spnc_hip

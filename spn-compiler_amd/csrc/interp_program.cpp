@@ -1,6 +1,6 @@
 #include "interp_program.h"
 
-#include "emit_hip.h"
+#include "math_tables.h"
 
 #include <algorithm>
 #include <cmath>
