@@ -349,6 +349,37 @@ def test_packed_rows_on_the_discrete_configuration(native, variant, cfg):
     assert all(np.isneginf(got[r]) for r in (5, 6, 7, 8, 9)) and np.isfinite(got[10])
 
 
+@pytest.mark.parametrize("opts", [{}, {"hip-prefetch-rows": "false"}, {"hip-hoist-feature-values": "false"}, {"hip-fused-batch": 0}],
+                         ids=["default", "no-prefetch", "no-hoist", "unbatched"])
+def test_packed_rows_with_long_tables(native, opts):
+    """One sum over nine products of 32 categorical leaves, one feature with 120 categories: the padding that would make
+    unclamped packed bytes safe is too large here, so the kernel clamps every byte to its table's length (a minimum
+    written into one byte of the register, with the wait state that such a partial write needs). Inputs outside the
+    ranges, next to them and far away, give log 0."""
+    from spnc.structure import Categorical, Product, Sum
+    rng = np.random.default_rng(17)
+    domains = [120] + [int(d) for d in rng.integers(2, 7, 31)]
+    products = []
+    for _ in range(9):
+        products.append(Product(children=[Categorical(p=[float(v) for v in rng.dirichlet(np.ones(d))], scope=f) for f, d in enumerate(domains)]))
+    spn = Sum([float(v) for v in rng.dirichlet(np.ones(9))], products)
+    X = np.column_stack([rng.integers(0, d, 3000) for d in domains]).astype(np.int32)
+    X[3, 0] = 120
+    X[4, 0] = 127
+    X[5, 0] = 128
+    X[6, 0] = 255
+    X[7, 0] = 256
+    X[8, 5] = domains[5]
+    X[9, 31] = 2 ** 31 - 1
+    X[10, :] = [d - 1 for d in domains]
+    k = compile_spn(native, spn, "int32", marginal=False, **dict(opts, **{"hip-packed-rows": "true"}))
+    src = k.source()
+    assert "unsigned PK0 = R[0]" in src and "v_min_u32_sdwa %0, %0, %1 dst_sel:BYTE_0" in src   # packed rows, bytes clamped
+    got = run(k, X)
+    check_f32(got, oracle_model(spn, "int32"), X, False)
+    assert all(np.isneginf(got[r]) for r in range(3, 10)) and np.isfinite(got[10]) and np.isfinite(got[:3]).all()
+
+
 @pytest.mark.parametrize("dtype,marginal", [("uint8", False), ("int32", False), ("float32", True), ("float64", True)])
 def test_grouped_tables_feature_types_and_marginals(native, dtype, marginal):
     """Small graph, grouping forced: every feature has five or six table leaves (one index each), joint tables for the
