@@ -505,22 +505,30 @@ struct Emitter {
       std::vector<std::string> adds;
       for (size_t q = b0; q < std::min(G.units.size(), b0 + batch); ++q) {
         const FusedUnit& u = G.units[q];
-        // Byte offset of the unit's entry: (a * rowsB + b) * stride * sizeof(real_t), one multiply per feature.
-        std::string idx = packedByteTimes(u.fa, size_t(u.rowsB) * u.stride * realBytes);
+        // LDS address of the unit's entry: table + (a * rowsB + b) * stride * sizeof(real_t), as one statement of two
+        // or three instructions: a multiply per feature that takes its byte straight out of the packed register, and
+        // an add that brings in the table's address, so that every read of the unit is this register plus a
+        // constant offset. (Left to the compiler, the address of nearly every read got an add of its own.)
+        const std::string idx = "a" + std::to_string(extractions2++);
+        const std::string sel = " dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:";
+        const size_t unitBytes = size_t(u.base) * realBytes;
         if (u.fb != UINT32_MAX) {
-          const std::string second = packedByteTimes(u.fb, u.stride * realBytes);
-          const std::string joint = "j" + std::to_string(extractions2++);
-          body << "  const unsigned " << joint << " = " << idx << " + " << second << ";\n";
-          idx = joint;
+          body << "  unsigned " << idx << ", " << idx << "b;\n  asm volatile(\"v_mul_u32_u24_sdwa %0, %2, %4" << sel << byteSel(u.fa) << " src1_sel:DWORD\\n\\t"
+               << "v_mul_u32_u24_sdwa %1, %3, %5" << sel << byteSel(u.fb) << " src1_sel:DWORD\\n\\tv_add3_u32 %0, %0, %1, %6\" : \"=&v\"(" << idx << "), \"=&v\"("
+               << idx << "b) : \"v\"(PK" << u.fa / 4 << "), \"v\"(PK" << u.fb / 4 << "), \"s\"(" << size_t(u.rowsB) * u.stride * realBytes << "u), \"s\"("
+               << u.stride * realBytes << "u), \"s\"(spn_tab_lds + " << unitBytes << "u));\n";
+        } else {
+          body << "  unsigned " << idx << ";\n  asm volatile(\"v_mul_u32_u24_sdwa %0, %1, %2" << sel << byteSel(u.fa) << " src1_sel:DWORD\\n\\tv_add_u32 %0, %3, %0\" : \"=&v\"("
+               << idx << ") : \"v\"(PK" << u.fa / 4 << "), \"s\"(" << u.stride * realBytes << "u), \"s\"(spn_tab_lds + " << unitBytes << "u));\n";
         }
         for (size_t j = 0; j < k; j += 2) {
           const std::string r = "r" + std::to_string(extractions2++);
-          const std::string address = "reinterpret_cast<const char*>(tab + " + std::to_string(u.base + j) + "u) + " + idx;
+          const std::string address = idx + " + " + std::to_string(j * realBytes) + "u";
           if (u.stride == 1) {
-            body << "  const real_t " << r << " = *reinterpret_cast<const real_t*>(" << address << ");\n";
+            body << "  const real_t " << r << " = *reinterpret_cast<const __attribute__((address_space(3))) real_t*>(" << address << ");\n";
             adds.push_back("  " + next(j) + " += " + r + ";\n");
           } else {
-            body << "  const spn_r2 " << r << " = *reinterpret_cast<const spn_r2*>(" << address << ");\n";
+            body << "  const spn_r2 " << r << " = *reinterpret_cast<const __attribute__((address_space(3))) spn_r2*>(" << address << ");\n";
             adds.push_back("  " + next(j) + " += " + r + "[0];\n");
             if (j + 1 < k) adds.push_back("  " + next(j + 1) + " += " + r + "[1];\n");
           }
@@ -1292,9 +1300,9 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
   e.midpointHook = prefetch;
   emitBody();
   if (prefetch)
-    s << "template <typename Mid>\nstatic __device__ __forceinline__ real_t spn_eval(const unsigned (&R)[SPN_F / 4], const real_t* __restrict__ tab, Mid&& spn_mid) {\n";
+    s << "template <typename Mid>\nstatic __device__ __forceinline__ real_t spn_eval(const unsigned (&R)[SPN_F / 4], const real_t* __restrict__ tab, unsigned spn_tab_lds, Mid&& spn_mid) {\n";
   else if (e.packedRows)
-    s << "static __device__ __forceinline__ real_t spn_eval(const unsigned (&R)[SPN_F / 4], const real_t* __restrict__ tab) {\n";
+    s << "static __device__ __forceinline__ real_t spn_eval(const unsigned (&R)[SPN_F / 4], const real_t* __restrict__ tab, unsigned spn_tab_lds) {\n";
   else if (e.vectorRows)
     s << "static __device__ __forceinline__ real_t spn_eval(const feat_t (&x)[SPN_F], const real_t* __restrict__ tab" << taskParams << ") {\n";
   else
@@ -1332,6 +1340,8 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
     s << "  __shared__ __attribute__((aligned(32))) real_t tab[SPN_NTAB];\n"
          "  for (unsigned t = threadIdx.x; t < SPN_NTAB; t += SPN_BLOCK) tab[t] = spn_tables[t];\n"
          "  __syncthreads();\n";
+    if (e.packedRows)  // the tables' address inside LDS, for reads addressed by plain integers
+      s << "  const unsigned spn_tab_lds = (unsigned)(unsigned long long)(__attribute__((address_space(3))) real_t*)tab;\n";
   } else if (js.tableEntries) {
     s << "  const real_t* tab = spn_tables;\n";
   } else {
@@ -1415,7 +1425,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
          "    if (big) {\n";
     issue(0, H, "      ");
     s << "    }\n"
-         "    const real_t value = spn_eval(R, tab, [&] {\n"
+         "    const real_t value = spn_eval(R, tab, spn_tab_lds, [&] {\n"
          "      if (big) {\n";
     stash(0, H, "        ");
     issue(H, Q - H, "        ");
@@ -1471,7 +1481,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
          "      if (SPN_Q & 1) R[SPN_Q - 1] = spn_pack4(x[SPN_F - 4], x[SPN_F - 3], x[SPN_F - 2], x[SPN_F - 1]);\n"
          "    }\n";
     if (e.packedRows) {
-      s << "    const real_t value = spn_eval(R, tab);\n";
+      s << "    const real_t value = spn_eval(R, tab, spn_tab_lds);\n";
     } else {
       s << "    feat_t x[SPN_F];\n"
            "#pragma unroll\n"
