@@ -346,16 +346,10 @@ struct Emitter {
 
   unsigned extractions2 = 0;
   static std::string byteSel(uint32_t f) { return "BYTE_" + std::to_string(f % 4); }
-  // Byte f of the packed row times a constant, as one instruction (the operand's byte select does the extraction).
+  // The byte of feature f as a value of its own.
   // Written as a volatile statement: these stay in program order, so an index exists only from where the generator
   // put it. Left to the compiler, the extractions are merged or moved to the top of the kernel, and hundreds of
   // indices stay in registers (measured: 256 registers and 470 spilled ones against 140).
-  std::string packedByteTimes(uint32_t f, size_t factor) {
-    const std::string name = "e" + std::to_string(extractions2++);
-    body << "  unsigned " << name << ";\n  asm volatile(\"v_mul_u32_u24_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:" << byteSel(f)
-         << " src1_sel:DWORD\" : \"=v\"(" << name << ") : \"v\"(PK" << f / 4 << "), \"s\"(" << factor << "u));\n";
-    return name;
-  }
   std::string packedByte(uint32_t f) {
     const std::string name = "e" + std::to_string(extractions2++);
     body << "  unsigned " << name << ";\n  asm volatile(\"v_bfe_u32 %0, %1, " << 8 * (f % 4) << ", 8\" : \"=v\"(" << name << ") : \"v\"(PK" << f / 4 << "));\n";

@@ -156,17 +156,30 @@ def _partition_example():
 
 @pytest.mark.parametrize("opts", [{}, {"hip-compute-type": "float64"}, {"use-log-space": "false"}, {"hip-sum-form": "pairwise", "hip-log2-domain": "false"}],
                          ids=["log-f32", "log-f64", "linear-f64", "strict-f32"])
-def test_reference_partitioning_example(native, opts):
-    """maxTaskSize=5 on the reference's seven-node example, as its tests run it: the graph becomes several kernels that
-    pass values through device memory, and the results are those of the uncut graph."""
+@pytest.mark.parametrize("size", [1, 2, 5])
+def test_reference_partitioning_example(native, opts, size):
+    """maxTaskSize=5 on the reference's seven-node example, as its tests run it (and the smallest bounds there are): the
+    graph becomes several kernels that pass values through device memory, and the results are those of the uncut graph."""
     rng = np.random.default_rng(30)
     X = np.column_stack((rng.integers(0, 2, 30), rng.integers(0, 2, 30))).astype("float64")
     spn = _partition_example()
-    k = compile_spn(native, spn, "float64", marginal=False, maxTaskSize=5, **opts)
+    k = compile_spn(native, spn, "float64", marginal=False, maxTaskSize=size, **opts)
     assert k.info()["num_tasks"] > 1
     got = run(k, X)
     ref = ev.ll_closed_f64(oracle_model(spn, "float64"), X, marginal=False)
     assert np.abs(got - ref).max() <= (F32_TOL if got.dtype == np.float32 else F64_TOL)
+
+
+@pytest.mark.parametrize("cfg,size", [("c1", 3), ("c2", 400), ("c3", 300), ("c5", 150), ("c5", 1200)])
+def test_partitioned_benchmark_configurations(native, cfg, size):
+    """The benchmark graphs cut into tasks: integer and float features, table leaves with their own LDS pool per task,
+    Gaussian leaves with missing values, sums split into trees where one sum alone exceeds the bound."""
+    from spnc import synthetic as syn
+    c = syn.CONFIGS[cfg]
+    spn, X = c["spn"](), c["inputs"](3000)
+    k = compile_spn(native, spn, c["dtype"], marginal=c["marginal"], maxTaskSize=size, **{"hip-kernel": "jit"})
+    assert k.info()["num_tasks"] > 1
+    check_f32(run(k, X), oracle_model(spn, c["dtype"]), X, c["marginal"])
 
 
 @pytest.mark.parametrize("size", [3, 10, 17])
