@@ -280,7 +280,7 @@ struct Emitter {
         for (const auto& u : G.units) t += fusedStride(G.products.size()) * size_t(u.rowsA) * u.rowsB;
       return t;
     };
-    const size_t budget = size_t(o.tableBudgetGiven ? o.tableBudgetKiB : 80) * 1024 / (f64 ? 8 : 4);
+    const size_t budget = size_t(o.tableBudgetGiven ? o.tableBudgetKiB : 96) * 1024 / (f64 ? 8 : 4);
     while (total() > budget) {
       FusedGroup* bestG = nullptr;
       size_t bestU = 0, bestGain = 0;

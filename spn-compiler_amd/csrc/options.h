@@ -41,7 +41,7 @@ struct CompileOptions {
   int tableGroupWindow = 96;                   // "hip-table-group-window": tables of a group are used within this many table uses of each other
   int tablePadKiB = 18;                        // "hip-table-pad-kib": LDS beyond the table budget that blocks of four columns may take (unused columns)
   int tableBudgetKiB = 62;                     // "hip-table-budget-kib": LDS the table pool may grow to when leaves are paired into joint tables
-  bool tableBudgetGiven = false;               // without the option, kernels on packed rows pair up to 80 KiB (measured on the 100-feature discrete graph: 0.75 ms against 0.78 ms at 62 KiB)
+  bool tableBudgetGiven = false;               // without the option, kernels on packed rows pair up to 96 KiB (measured on the 100-feature discrete graph: 0.78 ms at 62 KiB, 0.75 ms at 80, 0.74 ms at 96 with leaves over three categories in tables too)
   int jointMaxEntries = 160;                   // "hip-joint-max-entries": largest joint table (entries) a pair of table leaves may get
   int interpShortSlots = 0;                    // "hip-interp-short-slots": LDS value slots per lane the interpreter program aims for (0 = automatic)
   bool interpLeafRegions = true;               // "hip-interp-leaf-regions": Gaussian leaf products read by one matrix-form outer sum are computed inside it
@@ -53,7 +53,7 @@ struct CompileOptions {
   int interpStagedLong = -1;                   // "hip-interp-staged-features": lds|spill (-1 = automatic): tier of the staged input features
   long interpLongRange = -1;                   // "hip-interp-long-range": values living longer than this many instructions go to the long-lived pool (-1 = automatic)
   int packedRows = -1;                         // "hip-packed-rows": wide rows of small integer features stay packed four to a register and the table leaves of sibling products are evaluated together (1), not (0), decided per kernel (-1)
-  int oneHotMaxDomain = 3;                     // "hip-one-hot-max-domain": with packed rows, table leaves over at most this many categories are evaluated as multiply-adds on the vector unit instead of LDS reads
+  int oneHotMaxDomain = 2;                     // "hip-one-hot-max-domain": with packed rows, table leaves over at most this many categories are evaluated as multiply-adds on the vector unit instead of LDS reads
   bool nanMasks = true;                        // "hip-nan-masks": with marginalisation in log space, a Gaussian leaf of a missing (NaN) feature is zeroed by a bitwise AND with a per-feature mask instead of a select per leaf
   int taskBufferMiB = 1024;                    // "hip-task-buffer-mib": most device memory the values passing between the tasks of a partitioned graph may take; larger batches run in several passes
   int prefetchRows = -1;                       // "hip-prefetch-rows": with the per-wavefront transposed load, the loads of a wavefront's next 64 rows are issued before the current ones are evaluated and stay in registers meanwhile (-1 = with packed rows)

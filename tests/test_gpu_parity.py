@@ -314,10 +314,11 @@ def test_grouped_tables_on_the_discrete_configuration(native, variant, cfg):
 
 
 PACKED = {
-    "default": {},                                        # rows packed to bytes, sibling products fused, one-hot leaves up to 3 categories
+    "default": {},                                        # rows packed to bytes, sibling products fused, leaves over two categories as multiply-adds
     "unbatched": {"hip-fused-batch": 0},
     "batch-7": {"hip-fused-batch": 7},
     "all-lds": {"hip-one-hot-max-domain": 0},
+    "one-hot-3": {"hip-one-hot-max-domain": 3},           # leaves over three categories as quadratic polynomials
     "one-hot-5": {"hip-one-hot-max-domain": 5},
     "no-joint": {"hip-joint-tables": "false"},
     "small-budget": {"hip-table-budget-kib": 24},         # pairs are split again until the tables fit
