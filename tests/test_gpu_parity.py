@@ -496,6 +496,22 @@ def test_ragged_sizes(native, n):
         assert got.shape == (n,) and np.abs(got - full).max() <= F32_TOL
 
 
+def test_ragged_sizes_with_packed_rows(native):
+    """The per-wavefront transposed load with its prefetch: batches smaller than one wavefront's tile (nothing to
+    prefetch at all), exact tiles, one row more or less, partial last blocks."""
+    from spnc import synthetic as syn
+    c = syn.CONFIGS["c3"]
+    spn = c["spn"]()
+    k = compile_spn(native, spn, c["dtype"])
+    assert "unsigned PK0 = R[0]" in k.source()
+    X = c["inputs"](70000)
+    full = ev.ll_closed_f64(oracle_model(spn, c["dtype"]), X, marginal=False)
+    for n in (1, 2, 63, 64, 65, 127, 128, 511, 512, 513, 1000, 4096, 65535, 65536, 65537, 70000):
+        got = k.execute(n, X[:n])
+        assert got.shape == (n,) and np.abs(got - full[:n]).max() <= F32_TOL, n
+    os.remove(k.fileName())
+
+
 def test_empty_batch_and_reuse(native):
     from spnc import synthetic as syn
     k = compile_spn(native, syn.c1_spn(), "int32")
