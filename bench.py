@@ -79,6 +79,27 @@ def make_device_inputs(name, cfg, n, torch, device):
     return x
 
 
+_SUSTAINED = {}
+
+
+def sustained_issue_rate(f64):
+    """Lane-operations per second of independent v_add_f32 (v_fma_f64) chains on every SIMD, measured now, in this process,
+    for about half a second: what the vector units of this box sustain at the clock it holds under load. The published
+    peak is quoted at the nominal clock. None when the calibration library is not built."""
+    if f64 not in _SUSTAINED:
+        import ctypes
+        path = os.path.join(ROOT, "spn-compiler_amd", "libspnc_issue_rate.so")
+        rate = ctypes.c_double(0.0)
+        try:
+            lib = ctypes.CDLL(path)
+            lib.spnc_issue_rate.argtypes = [ctypes.c_int, ctypes.c_double, ctypes.POINTER(ctypes.c_double)]
+            ok = lib.spnc_issue_rate(1 if f64 else 0, 0.5, ctypes.byref(rate)) == 0
+        except OSError:
+            ok = False
+        _SUSTAINED[f64] = rate.value if ok else None
+    return _SUSTAINED[f64]
+
+
 def measure(name, n, steps, warmup, torch, device, extra_options=None, fast_inputs=False):
     from spnc import synthetic as syn
     from spnc.hip import HIPCompiler
@@ -164,6 +185,12 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None, fast_inpu
         "valu_issue_frac": round(t_min_valu / t_launch, 4),
         "hbm_frac": round(t_min_hbm / t_launch, 4),
     }
+    if not hbm_bound:
+        sustained = sustained_issue_rate(f64)
+        if sustained:
+            roof["sustained_issue_per_s"] = sustained                      # measured in this process, see sustained_issue_rate()
+            roof["sustained_over_published"] = round(sustained / valu_peak, 4)
+            roof["frac_of_sustained"] = round(slots * n / sustained / t_launch, 4)
     if f64:
         # A float64 exp or log is not one quarter-rate instruction as in float32 but a routine of its own: about 11
         # double-rate instructions and one LDS read here. Priced at that cost the same launch reads:
@@ -323,6 +350,9 @@ def main():
                 res["host_path"] = host_path(kernel, x_host, torch)
         if not args.no_cpu:
             res["cpu_baseline"] = cpu_baseline(res["workload"], cfg, spn, x_host)
+            if res.get("host_path") and res["cpu_baseline"]["value"] > 0:
+                # below 1: for data that starts in host memory, the host's own cores finish sooner than the trip over PCIe
+                res["host_path_vs_cpu_baseline"] = round(res["host_path"]["pageable_samples_per_s"] / res["cpu_baseline"]["value"], 3)
         os.remove(kernel.fileName())
         del kernel, x_host
         torch.cuda.empty_cache()
@@ -336,7 +366,8 @@ def main():
                 continue
             r = one(name)
             others[name] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()
-                            if k in ("samples_per_s", "n", "ms_per_step", "roofline", "nodes", "cpu_baseline", "host_path", "kernel_key")}
+                            if k in ("samples_per_s", "n", "ms_per_step", "roofline", "nodes", "cpu_baseline", "host_path", "kernel_key",
+                                     "compile_s", "host_path_vs_cpu_baseline")}
     line = {
         "metric": "samples/sec log-likelihood on 1 MI355X + % of HBM/FP32 roofline",
         "value": round(res["samples_per_s"], 1),
@@ -353,9 +384,11 @@ def main():
                  "synthetic (seeded NumPy generators for SPN parameters and inputs, the arrays of the parity tests; inputs resident in HBM "
                  "before the timed region)"),
         "config": {"workload": f"{args.config}: {res['desc']}", "samples": res["n"], "nodes": res["nodes"], "kernel_key": res["kernel_key"]},
+        "compile_s": res["compile_s"],      # compile_ll: serialise, build the graph, generate and hipRTC-compile the kernel (log_likelihood = this + execute)
         "roofline": res["roofline"],
         "cpu_baseline": res.get("cpu_baseline"),
         "host_path": res.get("host_path"),
+        "host_path_vs_cpu_baseline": res.get("host_path_vs_cpu_baseline"),
         "target": {"samples_per_s": 1e9, "on": "c1 at 64M rows", "device_resident_met": None, "host_path_met": None},
         "others": others,
     }

@@ -90,17 +90,21 @@ SPNC_HIP_API int spnc_hip_execute_device(spnc_hip_kernel* k, size_t n, const voi
 /* Allocation-free variant of spnc_hip_execute_device for interpreter kernels (compiled with "hip-kernel" =
  * "interpreter", or chosen for large graphs). It has no counterpart in the reference: it exists for callers that
  * cannot allocate device memory where they call it (code under HIP graph capture, tight serving loops, harnesses that
- * forbid hipMalloc). Same arguments and results as spnc_hip_execute_device; neither this call nor anything it
- * calls allocates or frees device or pinned memory. Every device buffer the kernel needs besides d_in and d_out
- * (instruction stream, leaf tables, staged-feature descriptors, spilled value slots) lies in one fixed array of
- * SPNC_HIP_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends. The first call
- * with a kernel on a device, and the first after another kernel used the array, copies the kernel's program into it
- * on `stream` from host memory (make that call outside graph capture); later calls only launch. The launch uses
- * as many blocks as have room for their spilled slots in the array, so large programs run with a smaller grid
+ * forbid hipMalloc). Same arguments and results as spnc_hip_execute_device; the library itself makes no hipMalloc,
+ * hipFree, hipHostMalloc or hipHostFree call on this path (what the HIP runtime does inside a launch or a copy is
+ * its own). Every device buffer the kernel needs besides d_in and d_out (instruction stream, leaf tables,
+ * staged-feature descriptors, spilled value slots) lies in one fixed array of SPNC_HIP_STATIC_SCRATCH_BYTES inside
+ * the library, one copy per GPU, held until the process ends. The first call with a kernel on a device, and the
+ * first after another kernel used the array, copies the kernel's program into it on `stream` from pageable host
+ * memory (make that call outside graph capture; the copy may block the host); later calls only launch. The launch
+ * uses as many blocks as have room for their spilled slots in the array, so large programs run with a smaller grid
  * than spnc_hip_execute_device would give them, with identical results. A program whose stream, tables and one
  * block's spilled slots exceed the array, and a straight-line kernel (loading its code object allocates), are
- * refused with an error. All calls on one GPU share the array: calls that overlap in time on one GPU race, from any
- * thread, stream or kernel handle; order them on one stream or with events. */
+ * refused with an error, and so is a call made with another device current than the kernel's first call saw. All
+ * calls on one GPU share the array, from any thread or kernel handle: a call on another stream than the previous
+ * call's waits for that call's kernel through an event (created when the array's address is resolved, i.e. on the
+ * process's first call on that GPU), so calls on several streams run one after the other instead of racing. Calls on
+ * a stream that is being captured into a graph are not ordered by the library: order such graphs' launches yourself. */
 #define SPNC_HIP_STATIC_SCRATCH_BYTES (64u << 20)
 SPNC_HIP_API int spnc_hip_execute_device_static(spnc_hip_kernel* k, size_t n, const void* d_in, void* d_out, void* stream);
 

@@ -1036,6 +1036,12 @@ unsigned pickVectorBytes(unsigned rowBytes, unsigned elemBytes) {
 
 }  // namespace
 
+// Whether the library's exp/log are inlined at every call: by the size of the graph and its call sites. In linear space
+// every Gaussian leaf is a call of the double-precision exp (1326 of them cost 80 s of hipRTC time inlined, 10 s out of line).
+bool inlineLibraryMath(const Graph& g, const CompileOptions& o) {
+  return g.nodes.size() + g.stats.sumTerms + (o.useLogSpace ? 0 : 3 * size_t(g.stats.gaussians)) <= 4000;
+}
+
 JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::string& entry) {
   Emitter e(g, o);
   // Short rows are fetched with the widest vector loads their size allows, all samples of a
@@ -1167,7 +1173,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
     s << "};\n";
   }
   // Out-of-line library math keeps hipRTC times in seconds for large graphs; small graphs inline it.
-  const bool inlineMath = o.inlineMath >= 0 ? o.inlineMath == 1 : g.nodes.size() + g.stats.sumTerms <= 4000;
+  const bool inlineMath = o.inlineMath >= 0 ? o.inlineMath == 1 : inlineLibraryMath(g, o);
   const char* mathAttr = inlineMath ? "__forceinline__" : "__attribute__((noinline))";
   if (e.log2Dom && e.f64) {
     // Base-2 exponential and logarithm in double for the arguments this kernel produces (exponents <= 0 up to

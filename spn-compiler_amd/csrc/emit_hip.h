@@ -34,4 +34,7 @@ struct JitSource {
 // read from and to write to, [rows][n] values of the kernel's compute type.
 JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::string& entry = "spn_kernel");
 
+// The automatic choice behind "hip-inline-math": true if the library's exp/log are inlined at every call of this graph.
+bool inlineLibraryMath(const Graph& g, const CompileOptions& o);
+
 }  // namespace spnc_hip

@@ -34,12 +34,16 @@ hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain
                              hipStream_t stream);
 
 // Device memory of the allocation-free entry point: one array per device inside the library's code object, held
-// from library load to process end. Returns its address on the current device and its size.
+// from library load to process end. Returns its address on the current device, its size and that device's ordinal.
+// The first call on a device also creates the event through which calls on different streams take turns on the
+// array (interpreterScratchEvent), so that no later call has anything left to create.
 constexpr size_t INTERP_SCRATCH_BYTES = size_t(64) << 20;
-hipError_t interpreterScratch(void** base, size_t* bytes);
+hipError_t interpreterScratch(void** base, size_t* bytes, int* device);
+hipEvent_t interpreterScratchEvent(int device);
 
-// Largest dynamic LDS size a block of the interpreter may request on the current device.
-hipError_t interpreterMaxLds(bool f64, bool log2Domain, size_t* bytes);
+// Largest LDS size a block may use on the current device, and the static LDS the kernel flavour for such a program
+// takes of it (the dynamic size a launch may request is the difference).
+hipError_t interpreterMaxLds(bool f64, bool log2Domain, uint32_t featureMode, size_t* bytes, size_t* staticBytes);
 
 // Resident blocks per CU for a given dynamic LDS size. featureMode: the program's (args.featureMode at launch);
 // float kernels are built once per feature mode.

@@ -38,9 +38,12 @@ namespace {
 static __device__ __align__(256) unsigned char scratch[INTERP_SCRATCH_BYTES];
 std::mutex scratchMutex;
 void* scratchAddress[64] = {};
+hipEvent_t scratchEvent[64] = {};
 }  // namespace
 
-hipError_t interpreterScratch(void** base, size_t* bytes) {
+hipEvent_t interpreterScratchEvent(int device) { return device >= 0 && device < 64 ? scratchEvent[device] : nullptr; }
+
+hipError_t interpreterScratch(void** base, size_t* bytes, int* device) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
@@ -50,22 +53,27 @@ hipError_t interpreterScratch(void** base, size_t* bytes) {
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return e;
+    e = hipEventCreateWithFlags(&scratchEvent[dev], hipEventDisableTiming);
+    if (e != hipSuccess) return e;
     scratchAddress[dev] = p;
   }
+  *device = dev;
   *base = scratchAddress[dev];
   *bytes = INTERP_SCRATCH_BYTES;
   return hipSuccess;
 }
 
-hipError_t interpreterMaxLds(bool f64, bool log2Domain, size_t* bytes) {
+hipError_t interpreterMaxLds(bool f64, bool log2Domain, uint32_t featureMode, size_t* bytes, size_t* staticBytes) {
   int dev = 0, maxLds = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   e = hipDeviceGetAttribute(&maxLds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev);
   if (e != hipSuccess) return e;
-  (void)f64;
-  (void)log2Domain;
+  hipFuncAttributes attr;
+  e = hipFuncGetAttributes(&attr, pick(f64, log2Domain, 1, featureMode));  // the three modes of a flavour hold the same static LDS
+  if (e != hipSuccess) return e;
   *bytes = size_t(maxLds);
+  *staticBytes = attr.sharedSizeBytes;
   return hipSuccess;
 }
 

@@ -156,7 +156,8 @@ class CopyCrew {
   }
   void copy(void* dst, const void* src, size_t bytes) {
     const size_t parts = workers_.size() + 1;
-    if (bytes < (size_t(4) << 20) || parts == 1) {
+    // A child process made by fork() inherits this object but not its threads: it copies on its own.
+    if (bytes < (size_t(4) << 20) || parts == 1 || getpid() != owner_) {
       std::memcpy(dst, src, bytes);
       return;
     }
@@ -183,7 +184,7 @@ class CopyCrew {
     const char* src = nullptr;
     size_t bytes = 0;
   };
-  CopyCrew() {
+  CopyCrew() : owner_(getpid()) {
     unsigned n = std::thread::hardware_concurrency();
     n = n >= 8 ? 3 : (n >= 4 ? 1 : 0);  // the calling thread copies a share too
     jobs_.resize(n);
@@ -207,6 +208,7 @@ class CopyCrew {
       }
     }
   }
+  const pid_t owner_;  // the process whose threads these are
   std::vector<std::thread> workers_;
   std::vector<Job> jobs_;
   std::mutex mutex_, callMutex_;
@@ -215,14 +217,30 @@ class CopyCrew {
   uint64_t generation_ = 0;
 };
 
-// True if `p` is host memory the GPU can copy from directly (hipHostMalloc / pinned), so that no staging copy is needed.
-bool isPinnedHost(const void* p) {
-  hipPointerAttribute_t attr;
-  if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
-    (void)hipGetLastError();  // ordinary pageable memory is "invalid value" to the runtime
+// True if the `bytes` bytes at `p` are host memory the GPU can copy from directly (hipHostMalloc / pinned), so that no
+// staging copy is needed: the first and the last byte must both lie in such an allocation.
+bool isPinnedHost(const void* p, size_t bytes) {
+  auto pinned = [](const void* q) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, q) != hipSuccess) {
+      (void)hipGetLastError();  // ordinary pageable memory is "invalid value" to the runtime
+      return false;
+    }
+    return attr.type == hipMemoryTypeHost;
+  };
+  return bytes != 0 && pinned(p) && pinned(static_cast<const char*>(p) + bytes - 1);
+}
+
+// Launches that share one device buffer take turns on it across streams: every launch records `done`, and a launch on
+// another stream than the last one waits for it first. Work on a stream that is being captured into a graph is left
+// alone (an event recorded outside the capture cannot be waited for inside it): the graph's own edges order it.
+bool capturing(hipStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
     return false;
   }
-  return attr.type == hipMemoryTypeHost;
+  return status != hipStreamCaptureStatusNone;
 }
 
 std::string makeKernelFilePath() {
@@ -292,7 +310,7 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
       // Whether the exp/log routines are inlined is decided by the size of the whole graph, as without the cut: what
       // costs hipRTC time is the sum of all inlined copies, whichever kernel they land in.
       CompileOptions taskOptions = o;
-      if (o.inlineMath < 0) taskOptions.inlineMath = g.nodes.size() + g.stats.sumTerms <= 4000 ? 1 : 0;
+      if (o.inlineMath < 0) taskOptions.inlineMath = inlineLibraryMath(g, o) ? 1 : 0;
       for (size_t t = 0; t < plan.tasks.size(); ++t) {
         const Graph& tg = plan.tasks[t];
         JitSource one = emitHipSource(tg, taskOptions, "spn_task" + std::to_string(t));
@@ -581,9 +599,12 @@ void Kernel::queryDevice() {
     // Value slots in LDS: as many as the program needs, capped so that two blocks fit a CU.
     int ldsPerCU = 0;
     hipCheck(hipDeviceGetAttribute(&ldsPerCU, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, device_), "LDS size query");
-    size_t maxBlock = 0;
-    hipCheck(interpreterMaxLds(prog_.f64, prog_.log2Domain, &maxBlock), "LDS limit query");
+    // The kernel's own static LDS (the float64 log2 flavour keeps 4.7 KiB of exp2/log2 tables there) comes out of
+    // the same memory: without it in the sum a program of 40 slots would leave room for one block per CU, not two.
+    size_t maxBlock = 0, staticLds = 0;
+    hipCheck(interpreterMaxLds(prog_.f64, prog_.log2Domain, prog_.featureMode, &maxBlock, &staticLds), "LDS limit query");
     size_t budget = std::min<size_t>(maxBlock, size_t(ldsPerCU) / 2);
+    budget = budget > staticLds ? budget - staticLds : 0;
     uint32_t cap = uint32_t(budget / (INTERP_BLOCK * rb));
     if (prog_.ldsSlotLimit) cap = std::min(cap, prog_.ldsSlotLimit);
     if (prog_.numSlots <= cap) {
@@ -659,7 +680,10 @@ void Kernel::prepareDevice() {
     }
     const size_t lanes = size_t(numCUs_) * blocksPerCU_ * INTERP_BLOCK;
     spillBytes_ = size_t(prog_.numSlots - ldsSlots_) * lanes * rb;
-    if (spillBytes_) hipCheck(hipMalloc(&dSpill_, spillBytes_), "hipMalloc(spill)");
+    if (spillBytes_) {
+      hipCheck(hipMalloc(&dSpill_, spillBytes_), "hipMalloc(spill)");
+      hipCheck(hipEventCreateWithFlags(&spillTurn_.done, hipEventDisableTiming), "hipEventCreate");
+    }
   }
 }
 
@@ -684,6 +708,7 @@ void Kernel::releaseDevice() {
   dTables_ = nullptr;
   dStaged_ = nullptr;
   dSpill_ = nullptr;
+  spillTurn_.reset();
   if (dInter_) (void)hipFree(dInter_);
   dInter_ = nullptr;
   interRows_ = 0;
@@ -749,8 +774,30 @@ void Kernel::launch(size_t n, const void* dIn, void* dOut, hipStream_t stream) {
     void* args[] = {(void*)&dIn, (void*)&dOut, (void*)&n64};
     hipCheck(hipModuleLaunchKernel(function_, grid, 1, 1, blockSize_, 1, 1, 0, stream, args, nullptr), "kernel launch");
   } else {
+    // Every launch of this handle uses the one spill buffer: launches on different streams take turns.
+    const bool ordered = dSpill_ && !capturing(stream);
+    if (ordered) spillTurn_.wait(stream);
     launchProgram(n, dIn, dOut, dCode_, dTables_, dStaged_, dSpill_, size_t(numCUs_) * blocksPerCU_, stream);
+    if (ordered) spillTurn_.record(stream);
   }
+}
+
+void Turn::wait(hipStream_t stream) {
+  if (used && stream != last) hipCheck(hipStreamWaitEvent(stream, done, 0), "hipStreamWaitEvent");
+}
+
+void Turn::record(hipStream_t stream) {
+  if (!done) hipCheck(hipEventCreateWithFlags(&done, hipEventDisableTiming), "hipEventCreate");
+  hipCheck(hipEventRecord(done, stream), "hipEventRecord");
+  last = stream;
+  used = true;
+}
+
+void Turn::reset() {
+  if (done) (void)hipEventDestroy(done);
+  done = nullptr;
+  last = nullptr;
+  used = false;
 }
 
 void Kernel::launchProgram(size_t n, const void* dIn, void* dOut, const uint32_t* code, const void* tables, const uint32_t* staged,
@@ -785,6 +832,7 @@ void Kernel::executeDevice(size_t n, const void* dIn, void* dOut, hipStream_t st
 namespace {
 std::mutex g_scratchMutex;
 uint64_t g_scratchOwner[64] = {};   // per device: id of the kernel whose program the scratch array holds (0 = none)
+Turn g_scratchTurn[64];             // per device: calls on different streams take turns on the array
 std::atomic<uint64_t> g_nextKernelId{1};
 size_t roundUp256(size_t v) { return (v + 255) / 256 * 256; }
 }  // namespace
@@ -806,7 +854,10 @@ void Kernel::executeDeviceStatic(size_t n, const void* dIn, void* dOut, hipStrea
   if (!kernelId_) kernelId_ = g_nextKernelId.fetch_add(1);
   void* base = nullptr;
   size_t capacity = 0;
-  hipCheck(interpreterScratch(&base, &capacity), "hipGetSymbolAddress(scratch)");
+  int dev = -1;
+  hipCheck(interpreterScratch(&base, &capacity, &dev), "hipGetSymbolAddress(scratch)");
+  if (dev != device_)
+    fatal("RUNTIME ERROR: the kernel was set up on device " + std::to_string(device_) + ", the current device is " + std::to_string(dev));
   const size_t rb = prog_.f64 ? 8 : 4;
   const size_t codeAt = 0, tablesAt = roundUp256(codeImage_.size() * 4), stagedAt = tablesAt + roundUp256(tableImage_.size()),
                spillAt = stagedAt + roundUp256(stagedImage_.size() * 4);
@@ -817,22 +868,29 @@ void Kernel::executeDeviceStatic(size_t n, const void* dIn, void* dOut, hipStrea
   size_t maxBlocks = size_t(numCUs_) * blocksPerCU_;
   if (spillPerBlock) maxBlocks = std::min(maxBlocks, (capacity - spillAt) / spillPerBlock);
   char* p = static_cast<char*>(base);
-  {
-    std::lock_guard<std::mutex> scratchLock(g_scratchMutex);
-    if (device_ < 0 || device_ >= 64) fatal("RUNTIME ERROR: device ordinal out of range");
-    if (g_scratchOwner[device_] != kernelId_) {
-      g_scratchOwner[device_] = 0;  // stays "nobody's" if an upload fails half way
-      hipCheck(hipMemcpyAsync(p + codeAt, codeImage_.data(), codeImage_.size() * 4, hipMemcpyHostToDevice, stream), "program upload");
-      if (!tableImage_.empty())
-        hipCheck(hipMemcpyAsync(p + tablesAt, tableImage_.data(), tableImage_.size(), hipMemcpyHostToDevice, stream), "table upload");
-      if (!stagedImage_.empty())
-        hipCheck(hipMemcpyAsync(p + stagedAt, stagedImage_.data(), stagedImage_.size() * 4, hipMemcpyHostToDevice, stream), "staged upload");
-      g_scratchOwner[device_] = kernelId_;
-    }
+  // The array is shared by every kernel handle, thread and stream of the process on this device: the lock covers the
+  // whole enqueue, and a call on another stream than the previous one waits for that one's kernel first (its program
+  // and spilled values are still in use until then). The event was created when the array's address was resolved.
+  std::lock_guard<std::mutex> scratchLock(g_scratchMutex);
+  Turn& turn = g_scratchTurn[dev];
+  const bool ordered = !capturing(stream);
+  if (ordered) turn.wait(stream);
+  if (g_scratchOwner[dev] != kernelId_) {
+    g_scratchOwner[dev] = 0;  // stays "nobody's" if an upload fails half way
+    hipCheck(hipMemcpyAsync(p + codeAt, codeImage_.data(), codeImage_.size() * 4, hipMemcpyHostToDevice, stream), "program upload");
+    if (!tableImage_.empty())
+      hipCheck(hipMemcpyAsync(p + tablesAt, tableImage_.data(), tableImage_.size(), hipMemcpyHostToDevice, stream), "table upload");
+    if (!stagedImage_.empty())
+      hipCheck(hipMemcpyAsync(p + stagedAt, stagedImage_.data(), stagedImage_.size() * 4, hipMemcpyHostToDevice, stream), "staged upload");
+    g_scratchOwner[dev] = kernelId_;
   }
   launchProgram(n, dIn, dOut, reinterpret_cast<const uint32_t*>(p + codeAt), tableImage_.empty() ? nullptr : p + tablesAt,
                 stagedImage_.empty() ? nullptr : reinterpret_cast<const uint32_t*>(p + stagedAt), spillPerBlock ? p + spillAt : nullptr,
                 maxBlocks, stream);
+  if (ordered) {
+    turn.done = static_cast<hipEvent_t>(interpreterScratchEvent(dev));
+    turn.record(stream);
+  }
 }
 
 void Kernel::ensureStaging(size_t rows) {
@@ -872,7 +930,7 @@ void Kernel::execute(size_t n, const void* in, void* out) {
   ensureStaging(chunk);
   // Buffers the caller has pinned are copied from / to directly; pageable ones go through the pinned staging
   // buffers, filled by a few threads.
-  const bool pinnedIn = isPinnedHost(in), pinnedOut = isPinnedHost(out);
+  const bool pinnedIn = isPinnedHost(in, n * rowBytes), pinnedOut = isPinnedHost(out, n * bytesPerResult_);
   CopyCrew& crew = CopyCrew::instance();
   auto drain = [&](Stage& s) {
     if (!s.pendingRows) return;

@@ -22,6 +22,16 @@
 
 namespace spnc_hip {
 
+// Whose turn it is on a device buffer that launches on several streams share.
+struct Turn {
+  hipEvent_t done = nullptr;   // recorded after the last launch that used the buffer
+  hipStream_t last = nullptr;  // the stream of that launch
+  bool used = false;
+  void wait(hipStream_t stream);    // a launch on another stream than `last` waits for `done`
+  void record(hipStream_t stream);  // creates `done` on first use
+  void reset();
+};
+
 class Kernel {
  public:
   // Parses, validates and compiles a serialized query; writes the kernel file. Needs no GPU.
@@ -38,7 +48,7 @@ class Kernel {
   // Device buffers; enqueues on `stream` and returns.
   void executeDevice(size_t n, const void* dIn, void* dOut, hipStream_t stream);
   // The same for interpreter kernels without any allocation: the kernel's device buffers come out of the library's
-  // fixed scratch array (interp_kernel.h). Calls that overlap on one device race on that array.
+  // fixed scratch array (interp_kernel.h). Calls on different streams of one device take turns on that array.
   void executeDeviceStatic(size_t n, const void* dIn, void* dOut, hipStream_t stream);
 
  private:
@@ -100,6 +110,7 @@ class Kernel {
   uint32_t* dStaged_ = nullptr;
   void* dSpill_ = nullptr;
   size_t spillBytes_ = 0;
+  Turn spillTurn_;             // launches of this handle on different streams take turns on dSpill_
   uint32_t ldsSlots_ = 0;
   int interpMode_ = 0;
   size_t ldsBytes_ = 0;

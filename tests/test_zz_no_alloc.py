@@ -61,6 +61,32 @@ def test_static_entry_point_matches_the_allocating_one(native):
         os.remove(k.fileName())
 
 
+def test_static_entry_point_on_two_streams(native):
+    """Every call on a GPU shares the one scratch array: calls on different streams, here of two kernels that take the
+    array over from each other each time, wait for the call before them."""
+    import torch
+    from spnc import synthetic as syn
+    c4, c2 = syn.CONFIGS["c4"], syn.CONFIGS["c2"]
+    ka = compile_spn(native, c4["spn"](), c4["dtype"])
+    kb = compile_spn(native, c2["spn"](), c2["dtype"], **{"hip-kernel": "interpreter"})
+    n = 150_001
+    xa = torch.from_numpy(c4["inputs"](n)).cuda()
+    xb = torch.from_numpy(c2["inputs"](n)).cuda()
+    want_a = _device_run(ka.execute_device, xa, n, torch.float32)
+    want_b = _device_run(kb.execute_device, xb, n, torch.float32)
+    outs = [torch.full((n,), float("nan"), dtype=torch.float32, device="cuda") for _ in range(6)]
+    streams = [torch.cuda.Stream() for _ in range(2)]
+    torch.cuda.synchronize()
+    for rep in range(6):
+        k, x = (ka, xa) if rep % 2 == 0 else (kb, xb)
+        k.execute_device_static(n, x.data_ptr(), outs[rep].data_ptr(), streams[(rep // 2) % 2].cuda_stream if rep < 4 else streams[rep % 2].cuda_stream)
+    torch.cuda.synchronize()
+    for rep in range(6):
+        assert torch.equal(outs[rep], want_a if rep % 2 == 0 else want_b), rep
+    for k in (ka, kb):
+        os.remove(k.fileName())
+
+
 def test_static_entry_point_refuses_what_it_cannot_hold(native):
     import torch
     from spnc import synthetic as syn
