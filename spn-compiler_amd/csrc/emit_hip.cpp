@@ -47,6 +47,29 @@ struct Emitter {
   std::vector<uint32_t> useOrder, useRank;                          // tables in order of use; per table: its place in that order
   std::vector<uint32_t> featTableLen;  // per feature: longest table of any leaf on it (0 = none)
   std::vector<bool> featGauss;         // per feature: used by a Gaussian leaf
+  // float64 log-space kernels: a Gaussian leaf inside a product is den (x - mean)^2 + coef = A x^2 + B x + C, evaluated
+  // on per-feature x^2, x and 1 (all three zero for a missing feature) with one multiply-add per term, the constants as
+  // scalar operands: three double-rate instructions per leaf where subtract, square-and-shift, mask (two registers)
+  // and accumulate cost three double-rate and four single-rate ones; without marginalisation the C's of a product are
+  // one constant and a leaf costs two. The expansion cancels where x is near the mean: its absolute error is about
+  // 2^-52 |A| x^2 against 2^-52 |value| for the factored form, so it is used when, summed over the features, the
+  // worst leaf of each feature keeps that below 1e-11 for inputs within eight standard deviations of the mean.
+  bool expandedGauss = false;
+  // Where the constants of the expanded leaves come from. A double constant as a scalar operand takes two scalar moves
+  // with a literal each, and scalar instructions cost this kernel as much time as the multiply-adds they feed (measured:
+  // 4.0 ns per term with them, 2.0 ns without, three wavefronts per SIMD). Instead a vector register pair holds sixteen
+  // constants, lane l of every row of sixteen lanes the l-th (one coalesced 8-byte load per lane from a table in global
+  // memory), and v_fmac_f64 reads the one it wants through its cross-lane operand (DPP row_newbcast:l), at the rate
+  // of the plain instruction. All multiply-adds of a product sit in one assembler statement.
+  bool laneConstants = false;
+  std::vector<double> kPool;           // sixteen constants per vector, in order of use
+  int kVectorsNamed = 0;               // vectors whose marker has been written into the body
+  // With marginalisation the constant terms of a product's leaves depend on which of its features are missing. For
+  // products of up to four expanded leaves the sum of the C's of the present features (plus the weight folded into the
+  // product) is read from a table of 2^k entries in LDS, indexed by the pattern of present features, and is the
+  // value the multiply-adds accumulate onto: one LDS read per product instead of one multiply-add per leaf.
+  std::vector<double> cTables;
+  std::map<std::vector<uint32_t>, std::string> patternNames;  // features of a product (in leaf order) -> variable with the pattern
   std::vector<bool> featUsed;
   std::vector<bool> featPrepared;
   std::vector<bool> emitted;
@@ -124,7 +147,23 @@ struct Emitter {
     return comb(l, r);
   }
 
+  bool decideExpandedGauss() const {
+    if (!(f64 && logSpace && log2Dom) || o.gaussExpanded == 0) return false;
+    if (o.gaussExpanded == 1) return true;
+    std::vector<double> worst(g.numFeatures, 0.0);
+    for (const auto& n : g.nodes) {
+      if (n.kind != NodeKind::Gaussian) continue;
+      const double reach = std::fabs(n.mean) / n.stddev + 8.0;  // |x| / stddev at eight standard deviations
+      worst[n.feature] = std::max(worst[n.feature], 0x1p-52 * 3.0 * 0.5 * scale * reach * reach);
+    }
+    double sum = 0.0;
+    for (double w : worst) sum += w;
+    return sum <= 1e-11;
+  }
+
   void prepare() {
+    expandedGauss = decideExpandedGauss();
+    laneConstants = expandedGauss && o.laneConstants;
     featTableLen.assign(g.numFeatures, 0);
     featGauss.assign(g.numFeatures, false);
     featUsed.assign(g.numFeatures, false);
@@ -665,6 +704,10 @@ struct Emitter {
       std::stable_sort(kv.second.begin(), kv.second.end(), [&](uint32_t x, uint32_t y) { return useRank[x] < useRank[y]; });
     body.str("");
     body.clear();
+    kPool.clear();
+    kVectorsNamed = 0;
+    cTables.clear();
+    patternNames.clear();
     std::fill(emitted.begin(), emitted.end(), false);
     std::fill(featPrepared.begin(), featPrepared.end(), false);
     foldedWeight.clear();
@@ -757,6 +800,15 @@ struct Emitter {
         x = "x" + std::to_string(f);
       }
       if (featGauss[f]) body << "  const real_t g" << f << " = (real_t)" << x << ";\n";
+      if (featGauss[f] && expandedGauss) {
+        // x, x^2 and 1 of the expanded leaves; a missing feature zeroes all three, and with them every leaf over it
+        if (g.supportMarginal)
+          body << "  const bool gn" << f << " = g" << f << " != g" << f << ";\n  const real_t gx" << f << " = gn" << f << " ? 0.0 : g" << f
+               << ";\n  const real_t go" << f << " = gn" << f << " ? 0.0 : 1.0;\n";
+        else
+          body << "  const real_t gx" << f << " = g" << f << ";\n";
+        body << "  const real_t gq" << f << " = gx" << f << " * gx" << f << ";\n";
+      }
       if (featGauss[f] && nanMasks()) {
         // All ones, or zero when the feature is missing. The empty assembler statement hides where the value came from:
         // otherwise the compiler turns every AND with it back into a select.
@@ -790,6 +842,10 @@ struct Emitter {
     return (log2Dom ? (f64 ? "spn_log2(" : "__builtin_amdgcn_logf(") : "spn_log(") + a + ")";
   }
   std::string maxOf(const std::string& a, const std::string& b) const {
+    // Values that come out of assembler statements (products with lane constants) are not known to be quieted NaNs to
+    // the compiler, which then puts a canonicalising v_max_f64 x, x in front of every maximum that takes them; the
+    // instruction itself has fmax semantics, so those kernels call it directly.
+    if (laneConstants) return "spn_max(" + a + ", " + b + ")";
     return std::string(f64 ? "__builtin_fmax(" : "__builtin_fmaxf(") + a + ", " + b + ")";
   }
 
@@ -846,6 +902,104 @@ struct Emitter {
     return ops;
   }
 
+  // Sixteen consecutive lanes of the constant pool for `values` (at most sixteen), all within one vector.
+  std::pair<unsigned, unsigned> allocLanes(const std::vector<double>& values) {
+    if (kPool.size() % 16 + values.size() > 16) kPool.resize((kPool.size() + 15) / 16 * 16, 0.0);
+    const unsigned at = unsigned(kPool.size());
+    kPool.insert(kPool.end(), values.begin(), values.end());
+    // The vector is loaded where the marker stands; the markers are replaced by the loads of later vectors once the
+    // whole body is there, so that a load is in flight for a few products before its first use.
+    for (; kVectorsNamed <= int(at / 16); ++kVectorsNamed) body << "/*KV" << kVectorsNamed << "*/\n";
+    return {at / 16, at % 16};
+  }
+
+  // The expanded leaves of product i on top of `rest` (the name of the sum of its other children, or empty).
+  void emitExpandedLeaves(uint32_t i, const std::vector<uint32_t>& leaves, const std::string& rest, double fold) {
+    const std::string p = "p" + std::to_string(i) + "_";
+    const char* fma = "__builtin_fma(";
+    const bool marginal = g.supportMarginal;
+    struct Term { std::string input; double k; };
+    std::string acc;
+    double constants = fold;  // what does not depend on the inputs: the folded weight, and every leaf's C without marginalisation
+    size_t chunk = 0;
+    for (size_t lo = 0; lo < leaves.size(); ++chunk) {
+      // Leaves in chunks: four when a pattern table holds their constant terms, eight otherwise (sixteen lanes, two or
+      // three constants per leaf; an assembler statement takes thirty operands).
+      const bool table = marginal && o.marginalTablesKiB > 0 && (cTables.size() + 16) * sizeof(double) <= size_t(o.marginalTablesKiB) * 1024;
+      const size_t hi = std::min(leaves.size(), lo + (table ? 4 : (marginal ? 5 : 8)));
+      std::vector<Term> terms;
+      std::vector<uint32_t> feats;
+      std::vector<double> cs;
+      for (size_t j = lo; j < hi; ++j) {
+        const auto& leaf = g.nodes[leaves[j]];
+        emitFeaturePrep(leaf.feature);
+        const std::string f = std::to_string(leaf.feature);
+        const double den = -(1.0 / (2.0 * leaf.stddev * leaf.stddev)) * scale;
+        const double coef = (-std::log(leaf.stddev) + -0.5 * std::log(2 * M_PI)) * scale;
+        terms.push_back({"gq" + f, den});
+        terms.push_back({"gx" + f, -2.0 * leaf.mean * den});
+        const double C = den * leaf.mean * leaf.mean + coef;
+        feats.push_back(leaf.feature);
+        cs.push_back(C);
+        if (!marginal) constants += C;
+        else if (!table) terms.push_back({"go" + f, C});
+      }
+      // What the multiply-adds accumulate onto.
+      const std::string a0 = p + "i" + std::to_string(chunk);
+      std::string start;
+      if (table) {
+        auto it = patternNames.find(feats);
+        if (it == patternNames.end()) {
+          const std::string name = "pm" + std::to_string(patternNames.size());
+          body << "  const unsigned " << name << " = ";
+          for (size_t q = 0; q < feats.size(); ++q) body << (q ? " | " : "") << "(gn" << feats[q] << " ? 0u : " << (1u << q) << "u)";
+          body << ";\n";
+          it = patternNames.emplace(feats, name).first;
+        }
+        const size_t base = cTables.size();
+        for (unsigned mask = 0; mask < (1u << feats.size()); ++mask) {
+          double sum = chunk == 0 ? fold : 0.0;
+          for (size_t q = 0; q < feats.size(); ++q)
+            if (mask >> q & 1u) sum += cs[q];
+          cTables.push_back(sum);
+        }
+        start = "SPN_CTAB[" + std::to_string(base) + "u + " + it->second + "]";
+        if (chunk == 0) constants = 0.0;
+      } else if (chunk == 0 && constants != 0.0) {
+        start = lit(constants);
+        constants = 0.0;
+      }
+      if (!acc.empty()) start = start.empty() ? acc : "(" + acc + " + " + start + ")";
+      if (!laneConstants) {
+        std::string cur = start;
+        for (size_t t = 0; t < terms.size(); ++t) {
+          const std::string name = p + "e" + std::to_string(chunk) + "_" + std::to_string(t);
+          if (cur.empty()) body << "  const real_t " << name << " = " << terms[t].input << " * " << lit(terms[t].k) << ";\n";
+          else body << "  const real_t " << name << " = " << fma << terms[t].input << ", " << lit(terms[t].k) << ", " << cur << ");\n";
+          cur = name;
+        }
+        acc = cur;
+      } else {
+        std::vector<double> ks;
+        for (const Term& t : terms) ks.push_back(t.k);
+        const auto where = allocLanes(ks);
+        body << "  real_t " << a0 << " = " << (start.empty() ? "0.0" : start) << ";\n";
+        body << "  asm(\"";
+        for (size_t t = 0; t < terms.size(); ++t)
+          body << (t ? "\\n\\t" : "") << "v_fmac_f64_dpp %0, %1, %" << t + 2 << " row_newbcast:" << where.second + t << " row_mask:0xf bank_mask:0xf";
+        body << "\"\n      : \"+v\"(" << a0 << ") : \"v\"(kv" << where.first << ")";
+        for (const Term& t : terms) body << ", \"v\"(" << t.input << ")";
+        body << ");\n";
+        acc = a0;
+      }
+      lo = hi;
+    }
+    std::string value = acc;
+    if (constants != 0.0) value = "(" + value + " + " + lit(constants) + ")";
+    if (!rest.empty()) value = "(" + value + " + " + rest + ")";
+    body << "  const real_t " << v(i) << " = " << value << ";\n";
+  }
+
   // Log-space product with Gaussian leaves folded in. A leaf's value coef + d*d*den (d = x - mean)
   // is rewritten den * (d*d + coef/den), so that leaf plus accumulation cost three instructions
   // whose constants are all literals: d = x - mean; t = fma(d, d, coef/den); acc = fma(t, den, acc).
@@ -869,6 +1023,10 @@ struct Emitter {
       body << "  const real_t " << acc << " = " << e << ";\n";
     }
     const char* fma = f64 ? "__builtin_fma(" : "__builtin_fmaf(";
+    if (expandedGauss && !leaves.empty()) {
+      emitExpandedLeaves(i, leaves, acc, fold);
+      return;
+    }
     for (size_t k = 0; k < leaves.size(); ++k) {
       const auto& leaf = g.nodes[leaves[k]];
       emitFeaturePrep(leaf.feature);
@@ -1198,23 +1356,37 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
     // The polynomial coefficients are read from LDS as well, once per kernel, and stay in registers: as literals
     // every use costs two register moves, since a double constant cannot be an operand of the instruction itself.
     // c5..c1 of exp2, then l7..l1 of log2.
-    s << "__device__ const real_t spn_poly[12] = {";
+    // Entry 12 is the rounding constant of exp2, 1.5 * 2^52: as a value read from memory it stays in a register pair;
+    // as a literal it would be moved into the destination of a multiply-add before every use.
+    s << "__device__ const real_t spn_poly[13] = {";
     for (int j = 0; j < 12; ++j) s << (j ? ", " : "") << e.lit(math[576 + j]);
-    s << "};\n";
+    s << ", 0x1.8p+52};\n";
     s << "#ifndef SPN_EXP2_TABLE\n__shared__ real_t spn_exp2_lds[64];\n__shared__ __attribute__((aligned(16))) real_t spn_log2_lds[512];\n"
-         "__shared__ real_t spn_poly_lds[12];\n"
+         "__shared__ real_t spn_poly_lds[13];\n"
          "#define SPN_EXP2_TABLE spn_exp2_lds\n#define SPN_LOG2_TABLE spn_log2_lds\n#define SPN_POLY spn_poly_lds\n#endif\n";
+    // n = rint(64 x) without a rounding or conversion instruction: 64 x + 1.5 * 2^52 has an ulp of 1, so the sum's low
+    // mantissa bits are n as an integer and the sum minus the constant is n as a double. 2^(n >> 6) goes into the table
+    // value's exponent field by an integer add on its upper half (T[j] lies in [1, 2): field 1023; arguments are cut off
+    // at -1023, where the field reaches 0 with T[0] = 1, i.e. exactly 0.0; between -1023 and -1022 the result is
+    // some subnormal below 2^-1022, against terms of a sum whose largest is 1). A NaN argument stays NaN through r.
     s << "static __device__ " << mathAttr << " real_t spn_exp2(real_t x) {\n"
-      << (g.supportMarginal ? "  x = __builtin_fmax(x, -1100.0);  // missing features are handled at the leaves: no NaN gets here\n"
-                            : "  x = x < -1100.0 ? -1100.0 : x;  // keeps NaN\n")
+      << (g.supportMarginal ? "  x = __builtin_fmax(x, -1023.0);  // missing features are handled at the leaves: no NaN gets here\n"
+                            : "  x = x < -1023.0 ? -1023.0 : x;  // keeps NaN\n")
       <<
-         "  const real_t n = __builtin_rint(x * 64.0), r = __builtin_fma(n, -0x1p-6, x);\n"
-         "  const int ni = (int)n;\n"
-         "  const real_t t = SPN_EXP2_TABLE[ni & 63];\n"
+         "  union { real_t d; unsigned w[2]; } s, t;\n"
+         "  const real_t magic = SPN_POLY[12];\n"
+         "  s.d = __builtin_fma(x, 64.0, magic);\n"
+         "  const int ni = (int)s.w[0];\n"
+         "  const real_t r = __builtin_fma(s.d - magic, -0x1p-6, x);\n"
+         "  t.d = SPN_EXP2_TABLE[ni & 63];\n"
+         "  // t.w[1] += (ni >> 6) << 20 as two 32-bit instructions; written as C the compiler makes it a 64-bit add with a zero lower half\n"
+         "  unsigned hi;\n"
+         "  asm(\"v_ashrrev_i32 %0, 6, %1\\n\\tv_lshl_add_u32 %0, %0, 20, %2\" : \"=&v\"(hi) : \"v\"(ni), \"v\"(t.w[1]));\n"
+         "  t.w[1] = hi;\n"
          "  real_t p = SPN_POLY[0];\n"
          "  p = __builtin_fma(p, r, SPN_POLY[1]);\n  p = __builtin_fma(p, r, SPN_POLY[2]);\n"
          "  p = __builtin_fma(p, r, SPN_POLY[3]);\n  p = __builtin_fma(p, r, SPN_POLY[4]);\n"
-         "  return __builtin_ldexp(__builtin_fma(t, p * r, t), ni >> 6);\n}\n";
+         "  return __builtin_fma(t.d, p * r, t.d);\n}\n";
     s << "static __device__ " << mathAttr << " real_t spn_log2(real_t x) {\n"
          "  union { real_t d; unsigned long long u; } c;\n  c.d = x;\n"
          "  const unsigned hi = (unsigned)(c.u >> 32);\n"
@@ -1234,6 +1406,9 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
     s << "static __device__ " << mathAttr << " real_t spn_exp(real_t x) { return " << (e.f64 ? "exp(x)" : "expf(x)") << "; }\n";
     s << "static __device__ " << mathAttr << " real_t spn_log(real_t x) { return " << (e.f64 ? "log(x)" : "logf(x)") << "; }\n";
   }
+  if (e.laneConstants)
+    s << "static __device__ __forceinline__ real_t spn_max(real_t a, real_t b) {\n"
+         "  real_t r;\n  asm(\"v_max_f64 %0, %1, %2\" : \"=v\"(r) : \"v\"(a), \"v\"(b));\n  return r;\n}\n";
   if (e.nanMasks())
     s << (e.f64 ? "static __device__ __forceinline__ real_t spn_mask(real_t v, unsigned m) {\n"
                   "  union { real_t d; unsigned w[2]; } c;\n  c.d = v;\n  c.w[0] &= m;\n  c.w[1] &= m;\n  return c.d;\n}\n"
@@ -1299,6 +1474,31 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
   const char* taskArgs = g.isTask ? ", ext + i, res + i, n" : "";
   e.midpointHook = prefetch;
   emitBody();
+  std::string bodyText = e.body.str();
+  if (!e.kPool.empty()) {
+    e.kPool.resize((e.kPool.size() + 15) / 16 * 16, 0.0);
+    s << "__device__ __attribute__((aligned(128))) const real_t spn_kpool[" << e.kPool.size() << "] = {";
+    for (size_t i = 0; i < e.kPool.size(); ++i) s << (i ? ", " : "") << (i % 4 == 0 ? "\n  " : "") << e.lit(e.kPool[i]);
+    s << "};\n";
+    // Vector v is loaded where the marker of vector v - 3 stands (the first three at the top of the body).
+    const int vectors = int(e.kPool.size() / 16), ahead = 3;
+    auto load = [&](int v) {
+      return "  const real_t kv" + std::to_string(v) + " = spn_kpool[" + std::to_string(v * 16) + "u + (threadIdx.x & 15u)];\n";
+    };
+    std::string top;
+    for (int v = 0; v < std::min(ahead, vectors); ++v) top += load(v);
+    for (int v = 0; v < vectors; ++v) {
+      const std::string marker = "/*KV" + std::to_string(v) + "*/\n";
+      const size_t at = bodyText.find(marker);
+      bodyText.replace(at, marker.size(), v + ahead < vectors ? load(v + ahead) : std::string());
+    }
+    bodyText = top + bodyText;
+  }
+  if (!e.cTables.empty()) {
+    s << "#define SPN_NCTAB " << e.cTables.size() << "\n__device__ const real_t spn_ctab[SPN_NCTAB] = {";
+    for (size_t i = 0; i < e.cTables.size(); ++i) s << (i ? ", " : "") << (i % 4 == 0 ? "\n  " : "") << e.lit(e.cTables[i]);
+    s << "};\n#ifndef SPN_CTAB\n__shared__ real_t spn_ctab_lds[SPN_NCTAB];\n#define SPN_CTAB spn_ctab_lds\n#endif\n";
+  }
   if (prefetch)
     s << "template <typename Mid>\nstatic __device__ __forceinline__ real_t spn_eval(const unsigned (&R)[SPN_F / 4], const real_t* __restrict__ tab, unsigned spn_tab_lds, Mid&& spn_mid) {\n";
   else if (e.packedRows)
@@ -1307,7 +1507,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
     s << "static __device__ __forceinline__ real_t spn_eval(const feat_t (&x)[SPN_F], const real_t* __restrict__ tab" << taskParams << ") {\n";
   else
     s << "static __device__ __forceinline__ real_t spn_eval(const feat_t* __restrict__ row, const real_t* __restrict__ tab" << taskParams << ") {\n";
-  s << e.body.str();
+  s << bodyText;
   std::string root = Emitter::v(g.root());
   if (e.packedRows) {
     s << "  const real_t spn_root = " << root << (e.log2Dom ? (e.f64 ? " * 0x1.62e42fefa39efp-1" : " * 0x1.62e43p-1f") : "") << ";\n"
@@ -1334,8 +1534,9 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
   if (e.log2Dom && e.f64)
     s << "  for (unsigned t = threadIdx.x; t < 64; t += SPN_BLOCK) spn_exp2_lds[t] = spn_exp2_table[t];\n"
          "  for (unsigned t = threadIdx.x; t < 512; t += SPN_BLOCK) spn_log2_lds[t] = spn_log2_table[t];\n"
-         "  if (threadIdx.x < 12) spn_poly_lds[threadIdx.x] = spn_poly[threadIdx.x];\n"
-         "  __syncthreads();\n";
+         "  if (threadIdx.x < 13) spn_poly_lds[threadIdx.x] = spn_poly[threadIdx.x];\n"
+      << (e.cTables.empty() ? "" : "  for (unsigned t = threadIdx.x; t < SPN_NCTAB; t += SPN_BLOCK) spn_ctab_lds[t] = spn_ctab[t];\n")
+      << "  __syncthreads();\n";
   if (js.tableEntries && js.tablesInLds) {
     s << "  __shared__ __attribute__((aligned(32))) real_t tab[SPN_NTAB];\n"
          "  for (unsigned t = threadIdx.x; t < SPN_NTAB; t += SPN_BLOCK) tab[t] = spn_tables[t];\n"
@@ -1438,15 +1639,25 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
   } else {
     s << "  for (unsigned long long base = blockIdx.x * tile; base < n; base += gridDim.x * tile) {\n";
   }
-  const char* tail =
-      "      for (int u = 0; u < SPN_U; ++u) {\n"
-      "        const unsigned long long i = base + (unsigned long long)u * SPN_BLOCK + threadIdx.x;\n"
-      "        if (i < n) {\n"
-      "          feat_t x[SPN_F];\n"
-      "          spn_load_row(in, i, x);\n"
-      "          out[i] = spn_eval(x, tab);\n"
+  // Kernels whose multiply-adds read constants from other lanes of their row (lane constants) keep every lane of a
+  // wavefront at work: a cross-lane operand taken from a lane that is switched off disables the instruction in the lane
+  // that reads it. The lanes past the batch's end evaluate its last row and do not store.
+  const bool allLanes = !e.kPool.empty();
+  const std::string tailText =
+      std::string("      for (int u = 0; u < SPN_U; ++u) {\n"
+                  "        const unsigned long long i = base + (unsigned long long)u * SPN_BLOCK + threadIdx.x;\n") +
+      (allLanes ? "        {\n"
+                  "          feat_t x[SPN_F];\n"
+                  "          spn_load_row(in, i < n ? i : n - 1, x);\n"
+                  "          const real_t value = spn_eval(x, tab);\n"
+                  "          if (i < n) out[i] = value;\n"
+                : "        if (i < n) {\n"
+                  "          feat_t x[SPN_F];\n"
+                  "          spn_load_row(in, i, x);\n"
+                  "          out[i] = spn_eval(x, tab);\n") +
       "        }\n"
       "      }\n";
+  const char* tail = tailText.c_str();
   if (prefetch) {
     // emitted above
   } else if (waveTile) {
@@ -1511,15 +1722,20 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
          "    } else {\n"
       << tail << "    }\n";
   } else if (U == 1) {
-    s << "    const unsigned long long i = base + threadIdx.x;\n"
-         "    if (i < n) {\n";
+    if (allLanes)
+      s << "    const unsigned long long row = base + threadIdx.x;\n"
+           "    const unsigned long long i = row < n ? row : n - 1;\n"
+           "    {\n";
+    else
+      s << "    const unsigned long long i = base + threadIdx.x;\n"
+           "    if (i < n) {\n";
     if (e.vectorRows)
       s << "      feat_t x[SPN_F];\n"
            "      spn_load_row(in, i, x);\n"
            "      const real_t value = spn_eval(x, tab" << taskArgs << ");\n";
     else
       s << "      const real_t value = spn_eval(in + i * SPN_F, tab" << taskArgs << ");\n";
-    if (!g.isTask || g.taskFinal) s << "      __builtin_nontemporal_store(value, out + i);\n";
+    if (!g.isTask || g.taskFinal) s << (allLanes ? "      if (row < n) " : "      ") << "__builtin_nontemporal_store(value, out + i);\n";
     else s << "      (void)value;\n";
     s << "    }\n";
   } else {

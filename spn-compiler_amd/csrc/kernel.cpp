@@ -320,7 +320,7 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
                std::to_string(valuesIn) + " values in, " + std::to_string(tg.taskOutputs.size()) + " values out" + (tg.taskFinal ? ", the result" : "") + "\n";
         all += "namespace spn_task_scope" + std::to_string(t) + " {\n" + one.source + "}  // task " + std::to_string(t) +
                "\n#undef SPN_LOAD\n#undef SPN_LOAD_TILE\n#undef SPN_F\n#undef SPN_BLOCK\n#undef SPN_U\n#undef SPN_NTAB\n#undef SPN_DOUBLE_TABLES\n"
-               "#undef SPN_EXP2_TABLE\n#undef SPN_LOG2_TABLE\n#undef SPN_POLY\n";
+               "#undef SPN_EXP2_TABLE\n#undef SPN_LOG2_TABLE\n#undef SPN_POLY\n#undef SPN_NCTAB\n#undef SPN_CTAB\n";
         Task task;
         task.entry = one.entry;
         task.blockSize = one.blockSize;

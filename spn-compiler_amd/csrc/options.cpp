@@ -96,6 +96,13 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       o.jitMaxOps = parseInt(key, val);
     } else if (key == "hip-nan-masks") {
       o.nanMasks = parseBool(val);
+    } else if (key == "hip-gauss-expanded") {
+      o.gaussExpanded = val == "auto" ? -1 : (parseBool(val) ? 1 : 0);
+    } else if (key == "hip-lane-constants") {
+      o.laneConstants = parseBool(val);
+    } else if (key == "hip-marginal-tables-kib") {
+      o.marginalTablesKiB = parseInt(key, val);
+      if (o.marginalTablesKiB < 0 || o.marginalTablesKiB > 60) throw std::runtime_error("hip-marginal-tables-kib must be in [0,60]");
     } else if (key == "hip-task-buffer-mib") {
       o.taskBufferMiB = parseInt(key, val);
       if (o.taskBufferMiB < 1 || o.taskBufferMiB > 65536) throw std::runtime_error("hip-task-buffer-mib must be in [1,65536]");

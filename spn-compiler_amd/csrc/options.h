@@ -55,6 +55,9 @@ struct CompileOptions {
   int packedRows = -1;                         // "hip-packed-rows": wide rows of small integer features stay packed four to a register and the table leaves of sibling products are evaluated together (1), not (0), decided per kernel (-1)
   int oneHotMaxDomain = 2;                     // "hip-one-hot-max-domain": with packed rows, table leaves over at most this many categories are evaluated as multiply-adds on the vector unit instead of LDS reads
   bool nanMasks = true;                        // "hip-nan-masks": with marginalisation in log space, a Gaussian leaf of a missing (NaN) feature is zeroed by a bitwise AND with a per-feature mask instead of a select per leaf
+  int gaussExpanded = -1;                      // "hip-gauss-expanded": float64 log-space kernels evaluate a Gaussian leaf inside a product as A x^2 + B x + C on per-feature x^2, x and 1 (zeroed for a missing feature): three multiply-adds per leaf and no mask, two without marginalisation (-1 = where the expansion keeps 1e-11, see emit_hip.cpp)
+  bool laneConstants = true;                   // "hip-lane-constants": expanded Gaussian leaves take their constants from vector registers that hold sixteen constants each, one per lane of a row, through the cross-lane broadcast operand of the multiply-add (false = scalar moves with literals)
+  int marginalTablesKiB = 40;                  // "hip-marginal-tables-kib": LDS for the tables from which expanded leaves of kernels with marginalisation read the sum of their constant terms by the pattern of missing features (0 = a third multiply-add per leaf instead)
   int taskBufferMiB = 1024;                    // "hip-task-buffer-mib": most device memory the values passing between the tasks of a partitioned graph may take; larger batches run in several passes
   int prefetchRows = -1;                       // "hip-prefetch-rows": with the per-wavefront transposed load, the loads of a wavefront's next 64 rows are issued before the current ones are evaluated and stay in registers meanwhile (-1 = with packed rows)
   bool hoistFeatureValues = true;              // "hip-hoist-feature-values": with packed rows, the values (and squares) of the features whose leaves are polynomials are computed once at the top of the kernel (false = again in every group of products that uses them: more arithmetic, fewer registers)

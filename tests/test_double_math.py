@@ -8,6 +8,7 @@ import subprocess
 import numpy as np
 
 from conftest import compile_spn
+from test_packed_rows_host import ASM, _statement
 
 
 def _routines(native, tmp_path, marginal=False):
@@ -24,7 +25,7 @@ def _routines(native, tmp_path, marginal=False):
     for name in ("spn_exp2", "spn_log2"):
         m = re.search(r"static __device__ \S+ real_t " + name + r"\(real_t x\) \{.*?\n\}\n", src, re.S)
         assert m, name
-        parts.append(re.sub(r"static __device__ \S+ ", "", m.group(0)))
+        parts.append(ASM.sub(_statement, re.sub(r"static __device__ \S+ ", "", m.group(0))))   # assembler statements as the C they stand for
     c = tmp_path / ("m%d.c" % marginal)
     c.write_text("typedef double real_t;\ntypedef _Bool bool;\n" + "".join(parts))
     so = tmp_path / ("m%d.so" % marginal)

@@ -12,7 +12,7 @@ import pytest
 
 from conftest import GOLDEN, compile_query, compile_spn, load_golden, model_as_query, oracle_model
 from oracle import evaluate as ev
-from test_packed_rows_host import ASM, CLANG, _statement, needs_clang
+from test_packed_rows_host import ASM, CLANG, _statement, lane_constants_on_the_host, needs_clang
 
 PRELUDE = """#include <cmath>
 #define __device__
@@ -21,13 +21,13 @@ PRELUDE = """#include <cmath>
 static inline float __builtin_amdgcn_exp2f(float x) { return exp2f(x); }
 static inline float __builtin_amdgcn_logf(float x) { return log2f(x); }
 """
-TABLES = "#define SPN_EXP2_TABLE spn_exp2_table\n#define SPN_LOG2_TABLE spn_log2_table\n#define SPN_POLY spn_poly\n"
+TABLES = "#define SPN_EXP2_TABLE spn_exp2_table\n#define SPN_LOG2_TABLE spn_log2_table\n#define SPN_POLY spn_poly\n#define SPN_CTAB spn_ctab\n"
 
 
 def _host_part(text, name, task):
     """Everything of one kernel's source before the kernel itself, plus a loop over samples around its evaluation function."""
     body = text[:text.index('extern "C" __global__')]
-    body = ASM.sub(_statement, body).replace("__builtin_amdgcn_sched_barrier(0);", "")
+    body = lane_constants_on_the_host(ASM.sub(_statement, body)).replace("__builtin_amdgcn_sched_barrier(0);", "")
     body = body.replace("__device__ __attribute__((aligned(32))) const real_t spn_tables", "alignas(32) const real_t spn_tables")
     assert "asm" not in body
     tab = "spn_tables" if "spn_tables[SPN_NTAB]" in body else "nullptr"
@@ -62,7 +62,7 @@ def host_kernel(source, info, tmp_path):
             inner = rest[:rest.rindex("}  // task")]
             text += TABLES + scope + "{\n" + _host_part(inner, "task%d" % t, True) + "}\n" + "".join(
                 "#undef %s\n" % m for m in ("SPN_LOAD", "SPN_LOAD_TILE", "SPN_F", "SPN_BLOCK", "SPN_U", "SPN_NTAB", "SPN_DOUBLE_TABLES",
-                                            "SPN_EXP2_TABLE", "SPN_LOG2_TABLE", "SPN_POLY"))
+                                            "SPN_EXP2_TABLE", "SPN_LOG2_TABLE", "SPN_POLY", "SPN_NCTAB", "SPN_CTAB"))
     cpp, so = tmp_path / "k.cpp", tmp_path / "k.so"
     cpp.write_text(text)
     subprocess.check_call([CLANG, "-O1", "-shared", "-fPIC", "-std=c++17", "-ffp-contract=fast", "-w", "-o", str(so), str(cpp)])
@@ -132,8 +132,14 @@ def test_golden_models_on_the_host(native, tmp_path, name, opts):
 @needs_clang
 @pytest.mark.parametrize("cfg,opts", [("c1", {}), ("c1", {"maxTaskSize": 3}), ("c2", {"hip-samples-per-lane": 1}), ("c2", {"maxTaskSize": 300}),
                                        ("c5", {}), ("c5", {"hip-compute-type": "float64"}), ("c5", {"hip-compute-type": "float64", "maxTaskSize": 150}),
-                                       ("c5", {"hip-compute-type": "float64", "hip-nan-masks": "false"}), ("c3", {"hip-packed-rows": "false", "maxTaskSize": 300})],
-                         ids=["c1", "c1-cut", "c2", "c2-cut", "c5", "c5-f64", "c5-f64-cut", "c5-f64-selects", "c3-cut"])
+                                       ("c5", {"hip-compute-type": "float64", "hip-nan-masks": "false"}), ("c3", {"hip-packed-rows": "false", "maxTaskSize": 300}),
+                                       ("c5", {"hip-compute-type": "float64", "hip-gauss-expanded": "false"}),
+                                       ("c5", {"hip-compute-type": "float64", "hip-lane-constants": "false"}),
+                                       ("c5", {"hip-compute-type": "float64", "hip-marginal-tables-kib": 0}),
+                                       ("c5", {"hip-compute-type": "float64", "hip-marginal-tables-kib": 3}),
+                                       ("c2", {"hip-compute-type": "float64"}), ("c2", {"hip-compute-type": "float64", "hip-lane-constants": "false"})],
+                         ids=["c1", "c1-cut", "c2", "c2-cut", "c5", "c5-f64", "c5-f64-cut", "c5-f64-selects", "c3-cut", "c5-f64-factored",
+                              "c5-f64-scalar-constants", "c5-f64-no-pattern-tables", "c5-f64-few-pattern-tables", "c2-f64", "c2-f64-scalar-constants"])
 def test_benchmark_graphs_on_the_host(native, tmp_path, cfg, opts):
     from spnc import synthetic as syn
     c = syn.CONFIGS[cfg]

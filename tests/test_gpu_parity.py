@@ -566,6 +566,25 @@ def test_ragged_sizes(native, n):
         assert got.shape == (n,) and np.abs(got - full).max() <= F32_TOL
 
 
+@pytest.mark.parametrize("cfg", ["c2", "c5"])
+def test_ragged_sizes_in_float64(native, cfg):
+    """float64 kernels whose Gaussian leaves read their constants from other lanes of their row of sixteen: a batch that ends
+    inside a row, inside a wavefront, or before the first row is full must not show (every lane stays at work, the ones
+    past the end on the last row). With and without marginalisation, one and several tasks."""
+    from spnc import synthetic as syn
+    c = syn.CONFIGS[cfg]
+    spn = c["spn"]()
+    X = c["inputs"](1300)
+    want = ev.ll_closed_f64(oracle_model(spn, c["dtype"]), X, marginal=c["marginal"])
+    for opts in ({}, {"maxTaskSize": 700, "hip-kernel": "jit"}, {"hip-samples-per-lane": 2}):
+        k = compile_spn(native, spn, c["dtype"], marginal=c["marginal"], **dict(opts, **{"hip-compute-type": "float64"}))
+        assert "row_newbcast" in k.source()
+        for n in (1, 7, 15, 16, 17, 63, 65, 255, 520, 991, 1000, 1300):
+            got = k.execute(n, X[:n])
+            assert got.shape == (n,) and np.abs(got - want[:n]).max() <= F64_TOL, (opts, n)
+        os.remove(k.fileName())
+
+
 def test_ragged_sizes_with_packed_rows(native):
     """The per-wavefront transposed load with its prefetch: batches smaller than one wavefront's tile (nothing to
     prefetch at all), exact tiles, one row more or less, partial last blocks."""

@@ -34,9 +34,19 @@ def _instruction(line, names):
     if not line or line.startswith("s_nop"):
         return ""
     op, rest = line.split(None, 1)
-    mods = dict(re.findall(r"(dst_sel|dst_unused|src0_sel|src1_sel):(\w+)", rest))
-    args = [a.strip() for a in re.sub(r"\s+(dst_sel|dst_unused|src0_sel|src1_sel):\w+", "", rest).split(",")]
+    mods = dict(re.findall(r"(dst_sel|dst_unused|src0_sel|src1_sel|row_newbcast):(\w+)", rest))
+    args = [a.strip() for a in re.sub(r"\s+(dst_sel|dst_unused|src0_sel|src1_sel|row_newbcast|row_mask|bank_mask):\w+", "", rest).split(",")]
     v = [_operand(a, names) for a in args]
+    if op == "v_fmac_f64_dpp":
+        # the first source comes from lane row_newbcast of the register's row: the host build holds such a register
+        # (sixteen constants, one per lane of a row) as a pointer to the sixteen values
+        return f"{v[0]} = __builtin_fma({v[1]}[{int(mods['row_newbcast'])}], {v[2]}, {v[0]});"
+    if op == "v_max_f64":
+        return f"{v[0]} = __builtin_fmax({v[1]}, {v[2]});"
+    if op == "v_ashrrev_i32":
+        return f"{v[0]} = (unsigned)((int)({v[2]}) >> {v[1]});"
+    if op == "v_lshl_add_u32":
+        return f"{v[0]} = (({v[1]}) << {v[2]}) + ({v[3]});"
     if op in ("v_mul_u32_u24_sdwa", "v_min_u32_sdwa"):
         a, b = _select(v[1], mods.get("src0_sel")), _select(v[2], mods.get("src1_sel"))
         value = f"(({a} & 0xffffffu) * ({b} & 0xffffffu))" if op.startswith("v_mul") else f"(({a}) < ({b}) ? ({a}) : ({b}))"
@@ -70,6 +80,12 @@ def _statement(m):
 
 
 ASM = re.compile(r'asm(?:\s+volatile)?\s*\((?P<text>(?:\s*"(?:[^"\\]|\\.)*")+)\s*(?::(?P<tail>(?:[^;()]|\((?:[^()]|\([^()]*\))*\))*))?\)\s*;')
+
+
+def lane_constants_on_the_host(body):
+    """Registers that hold sixteen constants, one per lane of a row (read through v_fmac_f64_dpp), become pointers to the
+    sixteen values in the constant table."""
+    return re.sub(r"const real_t (kv\d+) = spn_kpool\[(\d+)u \+ \(threadIdx\.x & 15u\)\];", r"const real_t* \1 = spn_kpool + \2;", body)
 
 
 def host_library(source, saturation, tmp_path, tag):
