@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstring>
 #include <map>
 #include <sstream>
 #include <stdexcept>
@@ -1175,7 +1176,10 @@ struct Emitter {
       for (size_t j = lo; j < hi; ++j) y.push_back(term(j));
       std::string cm = tree(
           0, y.size(), [&](size_t j) { return y[j]; }, [&](const std::string& a, const std::string& b) { return maxOf(a, b); });
-      std::string mNew = fresh(maxOf(lo == 0 ? cm : maxOf(m, cm), lowest));
+      // (float64 kernels with marginalisation: their exp2 turns the NaN of -inf - -inf into 0 by itself, so no floor.)
+      const bool floorNeeded = !(f64 && log2Dom && g.supportMarginal);
+      const std::string mRaw = lo == 0 ? cm : maxOf(m, cm);
+      std::string mNew = fresh(floorNeeded ? maxOf(mRaw, lowest) : mRaw);
       std::string part = tree(
           0, y.size(), [&](size_t j) { return expOf(y[j] + " - " + mNew); },
           [&](const std::string& a, const std::string& b) { return "(" + a + " + " + b + ")"; });
@@ -1348,8 +1352,17 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
     // the CPU against exp2/log2 of libm). The tables live in LDS, 4.5 KiB per block.
     s << "#define SPN_DOUBLE_TABLES 1\n";
     const std::vector<double> math = doubleMathTables();
-    s << "__device__ const real_t spn_exp2_table[64] = {";
-    for (int j = 0; j < 64; ++j) s << (j ? ", " : "") << (j % 4 == 0 ? "\n  " : "") << e.lit(math[j]);
+    // Entry j holds 2^(j/64) with j << 14 taken off its upper half, so that adding n << 14 (n = 64 q + j) puts q into the
+    // exponent field in one instruction: the j's cancel (modulo 2^32).
+    s << "__device__ const unsigned long long spn_exp2_table[64] = {";
+    for (int j = 0; j < 64; ++j) {
+      uint64_t bits;
+      std::memcpy(&bits, &math[j], 8);
+      bits = (bits & 0xffffffffull) | (uint64_t(uint32_t(bits >> 32) - (uint32_t(j) << 14)) << 32);
+      char hex[32];
+      std::snprintf(hex, sizeof(hex), "0x%016llxull", (unsigned long long)bits);
+      s << (j ? ", " : "") << (j % 4 == 0 ? "\n  " : "") << hex;
+    }
     s << "};\n__device__ const real_t spn_log2_table[512] = {";
     for (int j = 0; j < 512; ++j) s << (j ? ", " : "") << (j % 4 == 0 ? "\n  " : "") << e.lit(math[64 + j]);
     s << "};\n";
@@ -1361,7 +1374,7 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
     s << "__device__ const real_t spn_poly[13] = {";
     for (int j = 0; j < 12; ++j) s << (j ? ", " : "") << e.lit(math[576 + j]);
     s << ", 0x1.8p+52};\n";
-    s << "#ifndef SPN_EXP2_TABLE\n__shared__ real_t spn_exp2_lds[64];\n__shared__ __attribute__((aligned(16))) real_t spn_log2_lds[512];\n"
+    s << "#ifndef SPN_EXP2_TABLE\n__shared__ unsigned long long spn_exp2_lds[64];\n__shared__ __attribute__((aligned(16))) real_t spn_log2_lds[512];\n"
          "__shared__ real_t spn_poly_lds[13];\n"
          "#define SPN_EXP2_TABLE spn_exp2_lds\n#define SPN_LOG2_TABLE spn_log2_lds\n#define SPN_POLY spn_poly_lds\n#endif\n";
     // n = rint(64 x) without a rounding or conversion instruction: 64 x + 1.5 * 2^52 has an ulp of 1, so the sum's low
@@ -1373,15 +1386,15 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
       << (g.supportMarginal ? "  x = __builtin_fmax(x, -1023.0);  // missing features are handled at the leaves: no NaN gets here\n"
                             : "  x = x < -1023.0 ? -1023.0 : x;  // keeps NaN\n")
       <<
-         "  union { real_t d; unsigned w[2]; } s, t;\n"
+         "  union { real_t d; unsigned long long u; unsigned w[2]; } s, t;\n"
          "  const real_t magic = SPN_POLY[12];\n"
-         "  s.d = __builtin_fma(x, 64.0, magic);\n"
+         "  // s = 64 x + magic with the factor as a scalar operand: written as C the constant is copied into the destination of a v_fmac_f64 every time\n"
+         "  asm(\"v_fma_f64 %0, %1, %2, %3\" : \"=v\"(s.d) : \"v\"(x), \"s\"(64.0), \"v\"(magic));\n"
          "  const int ni = (int)s.w[0];\n"
          "  const real_t r = __builtin_fma(s.d - magic, -0x1p-6, x);\n"
-         "  t.d = SPN_EXP2_TABLE[ni & 63];\n"
-         "  // t.w[1] += (ni >> 6) << 20 as two 32-bit instructions; written as C the compiler makes it a 64-bit add with a zero lower half\n"
+         "  t.u = SPN_EXP2_TABLE[ni & 63];\n"
          "  unsigned hi;\n"
-         "  asm(\"v_ashrrev_i32 %0, 6, %1\\n\\tv_lshl_add_u32 %0, %0, 20, %2\" : \"=&v\"(hi) : \"v\"(ni), \"v\"(t.w[1]));\n"
+         "  asm(\"v_lshl_add_u32 %0, %1, 14, %2\" : \"=v\"(hi) : \"v\"(ni), \"v\"(t.w[1]));\n"
          "  t.w[1] = hi;\n"
          "  real_t p = SPN_POLY[0];\n"
          "  p = __builtin_fma(p, r, SPN_POLY[1]);\n  p = __builtin_fma(p, r, SPN_POLY[2]);\n"

@@ -19,7 +19,7 @@ def _routines(native, tmp_path, marginal=False):
     assert src.count("spn_exp2(") > 200 and src.count("spn_log2(") > 70 and "spn_exp(" not in src and "spn_log(" not in src
     parts = ["#define SPN_EXP2_TABLE spn_exp2_table\n#define SPN_LOG2_TABLE spn_log2_table\n#define SPN_POLY spn_poly\n"]
     for name in ("spn_exp2_table", "spn_log2_table", "spn_poly"):   # the kernel copies these into LDS; on the CPU they are read where they are
-        m = re.search(r"__device__ const real_t " + name + r"\[\d+\] = \{.*?\};\n", src, re.S)
+        m = re.search(r"__device__ const (?:real_t|unsigned long long) " + name + r"\[\d+\] = \{.*?\};\n", src, re.S)
         assert m, name
         parts.append(m.group(0).replace("__device__ ", "static "))
     for name in ("spn_exp2", "spn_log2"):

@@ -45,6 +45,8 @@ def _instruction(line, names):
         return f"{v[0]} = __builtin_fmax({v[1]}, {v[2]});"
     if op == "v_ashrrev_i32":
         return f"{v[0]} = (unsigned)((int)({v[2]}) >> {v[1]});"
+    if op == "v_fma_f64":
+        return f"{v[0]} = __builtin_fma({v[1]}, {v[2]}, {v[3]});"
     if op == "v_lshl_add_u32":
         return f"{v[0]} = (({v[1]}) << {v[2]}) + ({v[3]});"
     if op in ("v_mul_u32_u24_sdwa", "v_min_u32_sdwa"):
