@@ -591,25 +591,21 @@ __device__ __forceinline__ code_ptr leafRegionMatrixG(code_ptr ip, const Head& h
   return leafRegionMatrix<LOG2, SPILL, TIERED, STAGED, NA, NB, 4, true>(ip, h, wGlobal, fs, useRegs, regs, S);
 }
 
-// The matrix chain over ea[r] * eb[c] with the result kept in registers as a scaled vector: v = acc / max(acc);
-// returns log2(max(acc)).
-template <bool LOG2, int NA, int NB>
-__device__ __forceinline__ float scaledChain(const float* ea, const float* eb, const float (*A)[2], float* v) {
-  typedef Math<float, LOG2> Mt;
+// The matrix chain with the result left as it is: the linear sums, at most 1 each. For vectors that stay inside one
+// instruction; the program builder fuses sums only where the weights keep the largest entry of such a vector above 2^-90.
+template <int NA, int NB>
+__device__ __forceinline__ void rawChain(const float* ea, const float* eb, const float (*A)[2], float* v) {
   float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
   MatrixSteps<0, NA * NB, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
-  const float m = rmax(rmax(rmax(d0[0], d0[1]), rmax(d0[2], d0[3])), rmax(rmax(d1[0], d1[1]), rmax(d1[2], d1[3])));
-  const float inv = __builtin_amdgcn_rcpf(rmax(m, 0x1p-100f));
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    v[t] = d0[t] * inv;
-    v[4 + t] = d1[t] * inv;
+    v[t] = d0[t];
+    v[4 + t] = d1[t];
   }
-  return Mt::log(m);
 }
 
 // OP_LEAFPAIRMM: an 8x8 outer sum whose operand lists are the result vectors of two leaf regions (N x N products
-// of G Gaussian leaves each, eight sums each; N = 4 is what the program builder emits). The two vectors stay in registers as scaled vectors; all weights,
+// of G Gaussian leaves each, eight sums each; N = 4 is what the program builder emits). The two vectors stay in registers as they are; all weights,
 // features and constants of the three sums are requested at the start.
 template <bool LOG2, bool SPILL, bool TIERED, bool STAGED, int N, int G, bool MARGINAL>
 __device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, const float* wGlobal, const FeatureSource& fs,
@@ -642,8 +638,8 @@ __device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, c
 #pragma unroll
   for (int side = 0; side < 2; ++side) {
     float ea[N], eb[N];
-    const float lb = leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + side * RECS, x + side * 2 * G, ea, eb);
-    base += lb + scaledChain<LOG2, N, N>(ea, eb, side == 0 ? A1 : A2, side == 0 ? va : vb);
+    base += leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + side * RECS, x + side * 2 * G, ea, eb);
+    rawChain<N, N>(ea, eb, side == 0 ? A1 : A2, side == 0 ? va : vb);
   }
   matrixChainAndStore<LOG2, SPILL, 8, 8>(va, vb, AT, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
   return ip + 2 + M + 1 + 4 * G + 2 * RECS + 2 * KL * M + 64 * M;
@@ -701,7 +697,7 @@ __device__ __forceinline__ code_ptr leafQuadMatrix(code_ptr ip, const Head& h, c
       const int region = 2 * pair + side;
       float ea[N], eb[N];
       base += leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + region * RECS, x + region * 2 * G, ea, eb);
-      base += scaledChain<LOG2, N, N>(ea, eb, AL[region], v[side]);
+      rawChain<N, N>(ea, eb, AL[region], v[side]);
     }
     if (pair == 0) {
       loadLeaf(PAIRW, AL[2]);
@@ -710,7 +706,7 @@ __device__ __forceinline__ code_ptr leafQuadMatrix(code_ptr ip, const Head& h, c
     } else {
       loadTop(2 * PAIRW, ATOP);
     }
-    base += scaledChain<LOG2, 8, 8>(v[0], v[1], AT[pair], pv[pair]);
+    rawChain<8, 8>(v[0], v[1], AT[pair], pv[pair]);
   }
   matrixChainAndStore<LOG2, SPILL, 8, 8>(pv[0], pv[1], ATOP, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
   return ip + 2 + M + 1 + 8 * G + 4 * RECS + 2 * PAIRW + 64 * M;

@@ -557,7 +557,27 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       for (uint32_t s : instrs[k].srcs) fusedProduct[instrOfNode[s]] = true;
       instrs[k].srcs.clear();
     }
-    // Pairs of leaf regions: an 8x8 outer sum whose operand lists are the scaled result vectors of two leaf
+    // Inside a pair or a quad the result vectors of the inner sums stay in registers as they come out of the matrix
+    // chain, linear and not rescaled (a rescaling costs a maximum over eight values, a reciprocal, eight multiplies
+    // and a logarithm). That is safe while the vector's largest entry cannot underflow: the operand vectors' largest
+    // products are 1 (leaf regions: exp2(value - max)) or at least the product of the operands' floors, and the sum
+    // t that weighs this product most gets at least that weight of it. floorLog2 is log2 of this lower bound on
+    // max_t(result_t), from the weights alone; a fusion whose bound falls under 2^-90 is not made.
+    std::vector<double> floorLog2(instrs.size(), 0.0);
+    auto weightFloor = [&](uint32_t k) {
+      const std::vector<uint32_t>& sums = instrs[k].defs;
+      double low = INFINITY;
+      for (size_t q = 0; q < g.nodes[sums[0]].weights.size(); ++q) {
+        double best = 0.0;
+        for (uint32_t sNode : sums) best = std::max(best, g.nodes[sNode].weights[q]);
+        low = std::min(low, best);
+      }
+      return low > 0.0 ? std::log2(low) : -INFINITY;
+    };
+    for (uint32_t k = 0; k < instrs.size(); ++k)
+      if (leafRegion[k]) floorLog2[k] = weightFloor(k);
+    const double lowestFloor = -90.0;
+    // Pairs of leaf regions: an 8x8 outer sum whose operand lists are the result vectors of two leaf
     // regions of 4x4 products each, read by nothing else, takes them in: one instruction, the vectors stay in registers.
     for (uint32_t k = 0; k < instrs.size() && o.interpLeafRegions; ++k) {
       if (!matrixInstr[k] || leafRegion[k]) continue;
@@ -570,6 +590,8 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       const Outer& oi = outerOf.at(g.nodes[instrs[i].node].children);
       const Outer& oj = outerOf.at(g.nodes[instrs[j].node].children);
       if (oi.a.size() != 4 || oj.a.size() != 4 || g.nodes[oi.a[0]].children.size() != g.nodes[oj.a[0]].children.size()) continue;
+      floorLog2[k] = weightFloor(k) + floorLog2[i] + floorLog2[j];
+      if (!(floorLog2[k] >= lowestFloor)) continue;
       leafPair[k] = {i, j};
       fusedProduct[i] = fusedProduct[j] = true;
       instrs[k].srcs.clear();
@@ -589,6 +611,8 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
         return g.nodes[region.a[0]].children.size();
       };
       if (leavesOf(i) != leavesOf(j) || leavesOf(i) > 2) continue;
+      floorLog2[k] = weightFloor(k) + floorLog2[i] + floorLog2[j];
+      if (!(floorLog2[k] >= lowestFloor)) continue;
       leafQuad[k] = {i, j};
       fusedProduct[i] = fusedProduct[j] = true;
       instrs[k].srcs.clear();
