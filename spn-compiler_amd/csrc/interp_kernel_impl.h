@@ -24,6 +24,23 @@ namespace spnc_hip {
 
 namespace {
 
+// A wavefront that waits for memory between short bursts of arithmetic (leaf operands: constants, features, weights)
+// runs at a higher priority than one inside a long matrix chain, so that its bursts go out when its data arrive and
+// the chains of the other wavefronts fill the rest of the pipe.
+#ifndef SPN_PRIO
+#define SPN_PRIO 1
+#endif
+#if SPN_PRIO
+#ifndef SPN_PRIO_HIGH
+#define SPN_PRIO_HIGH 1
+#endif
+#define SPN_PRIO_LATENCY() __builtin_amdgcn_s_setprio(SPN_PRIO_HIGH)
+#define SPN_PRIO_CHAIN() __builtin_amdgcn_s_setprio(0)
+#else
+#define SPN_PRIO_LATENCY()
+#define SPN_PRIO_CHAIN()
+#endif
+
 #define SPN_CONST __attribute__((address_space(4)))
 typedef const SPN_CONST uint32_t* code_ptr;
 
@@ -396,7 +413,9 @@ __device__ __forceinline__ void matrixChainAndStore(const float* ea, const float
   typedef Math<float, LOG2> Mt;
   constexpr int M = 8, K = NA * NB;
   float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+  SPN_PRIO_CHAIN();
   MatrixSteps<0, K, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
+  SPN_PRIO_LATENCY();
   float res[M];
   if (outScaled) {
     // acc_t / max(acc) and one logarithm for the whole vector. All-zero accumulators (impossible evidence) give
@@ -596,7 +615,9 @@ __device__ __forceinline__ code_ptr leafRegionMatrixG(code_ptr ip, const Head& h
 template <int NA, int NB>
 __device__ __forceinline__ void rawChain(const float* ea, const float* eb, const float (*A)[2], float* v) {
   float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+  SPN_PRIO_CHAIN();
   MatrixSteps<0, NA * NB, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
+  SPN_PRIO_LATENCY();
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
     v[t] = d0[t];
