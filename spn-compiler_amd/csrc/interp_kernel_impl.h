@@ -289,6 +289,84 @@ __device__ __forceinline__ code_ptr outerSum(code_ptr ip, int na, const Slots<R,
   return w + long(na) * NB * M * RW;
 }
 
+// Outer sum of eight double sums with the weights held in lanes. A double multiply-add takes its first factor from
+// another lane of its row of sixteen at no cost (v_fmac_f64 with the DPP control row_newbcast; the float forms of that
+// operand run at half rate, the double ones do not), so a register pair that every lane loaded 8 bytes of (lane l of a
+// row the l-th of sixteen consecutive weights) feeds sixteen multiply-adds: the eight sums of two products, which is
+// how the weights of this instruction lie in the stream (product-major, eight sums each). No scalar loads, no
+// scalar operands; the vectors of operand row r + 1 are requested while row r is being added up.
+struct __attribute__((packed, aligned(4))) StreamDouble {  // a double in the instruction stream: at a multiple of four bytes
+  double value;
+};
+template <bool LOG2, bool SPILL, int NB>
+__device__ __forceinline__ code_ptr outerSumLaneWeights(code_ptr ip, int na, const StreamDouble* wGlobal, const Slots<double, SPILL>& S) {
+  typedef Math<double, LOG2> Mt;
+  constexpr int M = 8, V = NB / 2;  // vectors of sixteen weights per operand row
+  code_ptr dsts = ip + 2, as = dsts + M, bs = as + na;
+  double eb[NB];
+  double mb = -__builtin_huge_val();
+#pragma unroll
+  for (int c = 0; c < NB; ++c) {
+    eb[c] = S.rd(bs[c]);
+    mb = rmax(mb, eb[c]);
+  }
+  mb = rmax(mb, Mt::lowest());
+  const StreamDouble* wl = wGlobal + (threadIdx.x & 15u);
+  double W[2][V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) W[0][v] = wl[v * 16].value;
+#pragma unroll
+  for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(eb[c] - mb);
+  double ma = -__builtin_huge_val();
+#pragma unroll 8
+  for (int r = 0; r < na; ++r) ma = rmax(ma, S.rd(as[r]));
+  ma = rmax(ma, Mt::lowest());
+  double acc[M];
+#pragma unroll
+  for (int t = 0; t < M; ++t) acc[t] = 0.0;
+  // Two rows per round so that the two sets of vectors keep their registers.
+  for (int r = 0; r < na; r += 2) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int row = r + half;
+      // the next row's weights (past the last row: the words that follow the instruction, read and not used)
+#pragma unroll
+      for (int v = 0; v < V; ++v) W[half ^ 1][v] = wl[((row + 1) * V + v) * 16].value;
+      const double ea = Mt::exp(S.rd(as[row]) - ma);
+#pragma unroll
+      for (int c = 0; c < NB; ++c) {
+        const double e = ea * eb[c];
+        if (c % 2 == 0)
+          asm("v_fmac_f64_dpp %0, %8, %9 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %1, %8, %9 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %2, %8, %9 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %3, %8, %9 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %4, %8, %9 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %5, %8, %9 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %6, %8, %9 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %7, %8, %9 row_newbcast:7 row_mask:0xf bank_mask:0xf"
+              : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+              : "v"(W[half][c / 2]), "v"(e));
+        else
+          asm("v_fmac_f64_dpp %0, %8, %9 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %1, %8, %9 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %2, %8, %9 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %3, %8, %9 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %4, %8, %9 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %5, %8, %9 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %6, %8, %9 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+              "v_fmac_f64_dpp %7, %8, %9 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+              : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+              : "v"(W[half][c / 2]), "v"(e));
+      }
+    }
+  }
+  const double base = ma + mb;
+#pragma unroll
+  for (int t = 0; t < M; ++t) S.wr(dsts[t], base + Mt::log(acc[t]));
+  return bs + NB + long(na) * NB * M * 2;
+}
+
 // Outer sum of eight float sums on the matrix cores. One 4x4x1 instruction multiplies, in every
 // group of four lanes, four values of matrix A by four values of matrix B and accumulates the 16
 // products; with the A-broadcast controls (cbsz = 4, abid = b) all sixteen groups take A from
@@ -1009,6 +1087,15 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
   }
   // OP_OUTERSUM
   const uint32_t m = h.word(2);
+  if constexpr (sizeof(R) == 8) {
+    // eight double sums over an even number of operand rows: the weights come through lanes (every lane of a
+    // wavefront is at work here: idle lanes recompute the batch's last sample)
+    if (m == 8 && (nb == 8 || nb == 4) && na % 2 == 0) {
+      const StreamDouble* wGlobal = reinterpret_cast<const StreamDouble*>(codeGlobal + ((ip - code0) + 2 + 8 + na + nb));
+      if (nb == 8) return outerSumLaneWeights<LOG2, SPILL, 8>(ip, na, wGlobal, S);
+      return outerSumLaneWeights<LOG2, SPILL, 4>(ip, na, wGlobal, S);
+    }
+  }
   if (m == 8) return outerSumNB<R, LOG2, SPILL, 8>(ip, na, nb, S);
   if (m == 4) return outerSumNB<R, LOG2, SPILL, 4>(ip, na, nb, S);
   return outerSumNB<R, LOG2, SPILL, 2>(ip, na, nb, S);
