@@ -28,9 +28,10 @@ struct InterpLaunch {
 };
 
 // Enqueues the interpreter on `stream`. ldsBytes = ldsSlots * INTERP_BLOCK * sizeof(compute type).
+// linear: the program computes with probabilities (double), not logarithms.
 // mode 0: all slots in LDS; 1: the program's short pool in LDS, flagged instructions may touch the spill tier;
 // 2: any instruction may touch the spill tier.
-hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain, int mode, unsigned grid, size_t ldsBytes,
+hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain, bool linear, int mode, unsigned grid, size_t ldsBytes,
                              hipStream_t stream);
 
 // Device memory of the allocation-free entry point: one array per device inside the library's code object, held
@@ -43,10 +44,10 @@ hipEvent_t interpreterScratchEvent(int device);
 
 // Largest LDS size a block may use on the current device, and the static LDS the kernel flavour for such a program
 // takes of it (the dynamic size a launch may request is the difference).
-hipError_t interpreterMaxLds(bool f64, bool log2Domain, uint32_t featureMode, size_t* bytes, size_t* staticBytes);
+hipError_t interpreterMaxLds(bool f64, bool log2Domain, bool linear, uint32_t featureMode, size_t* bytes, size_t* staticBytes);
 
 // Resident blocks per CU for a given dynamic LDS size. featureMode: the program's (args.featureMode at launch);
 // float kernels are built once per feature mode.
-hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, uint32_t featureMode, size_t ldsBytes, int* blocksPerCU);
+hipError_t interpreterOccupancy(bool f64, bool log2Domain, bool linear, int mode, uint32_t featureMode, size_t ldsBytes, int* blocksPerCU);
 
 }  // namespace spnc_hip

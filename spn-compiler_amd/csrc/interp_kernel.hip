@@ -18,12 +18,14 @@ const void* interpKernel_f32_natural_staged(int mode);
 const void* interpKernel_f32_natural_registers(int mode);
 const void* interpKernel_f64(int mode);
 const void* interpKernel_f64_log2(int mode);
+const void* interpKernel_f64_linear(int mode);
 
 namespace {
 
 // float kernels exist once per feature mode: the fused leaf instructions are long, and a kernel that held both
 // of their forms would run the staged one slower (instruction fetch). double kernels decide at run time.
-const void* pick(bool f64, bool log2Domain, int mode, uint32_t featureMode) {
+const void* pick(bool f64, bool log2Domain, bool linear, int mode, uint32_t featureMode) {
+  if (linear) return interpKernel_f64_linear(mode);  // linear space computes in double, as the reference does
   if (f64) return log2Domain ? interpKernel_f64_log2(mode) : interpKernel_f64(mode);
   if (featureMode == FEAT_REGISTER) return log2Domain ? interpKernel_f32_log2_registers(mode) : interpKernel_f32_natural_registers(mode);
   if (featureMode == FEAT_STAGED) return log2Domain ? interpKernel_f32_log2_staged(mode) : interpKernel_f32_natural_staged(mode);
@@ -63,22 +65,22 @@ hipError_t interpreterScratch(void** base, size_t* bytes, int* device) {
   return hipSuccess;
 }
 
-hipError_t interpreterMaxLds(bool f64, bool log2Domain, uint32_t featureMode, size_t* bytes, size_t* staticBytes) {
+hipError_t interpreterMaxLds(bool f64, bool log2Domain, bool linear, uint32_t featureMode, size_t* bytes, size_t* staticBytes) {
   int dev = 0, maxLds = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   e = hipDeviceGetAttribute(&maxLds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev);
   if (e != hipSuccess) return e;
   hipFuncAttributes attr;
-  e = hipFuncGetAttributes(&attr, pick(f64, log2Domain, 1, featureMode));  // the three modes of a flavour hold the same static LDS
+  e = hipFuncGetAttributes(&attr, pick(f64, log2Domain, linear, 1, featureMode));  // the three modes of a flavour hold the same static LDS
   if (e != hipSuccess) return e;
   *bytes = size_t(maxLds);
   *staticBytes = attr.sharedSizeBytes;
   return hipSuccess;
 }
 
-hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, uint32_t featureMode, size_t ldsBytes, int* blocksPerCU) {
-  const void* fn = pick(f64, log2Domain, mode, featureMode);
+hipError_t interpreterOccupancy(bool f64, bool log2Domain, bool linear, int mode, uint32_t featureMode, size_t ldsBytes, int* blocksPerCU) {
+  const void* fn = pick(f64, log2Domain, linear, mode, featureMode);
   if (ldsBytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(ldsBytes));
     if (e != hipSuccess) return e;
@@ -86,9 +88,9 @@ hipError_t interpreterOccupancy(bool f64, bool log2Domain, int mode, uint32_t fe
   return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocksPerCU, fn, int(INTERP_BLOCK), ldsBytes);
 }
 
-hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain, int mode, unsigned grid, size_t ldsBytes,
+hipError_t launchInterpreter(const InterpLaunch& args, bool f64, bool log2Domain, bool linear, int mode, unsigned grid, size_t ldsBytes,
                              hipStream_t stream) {
-  const void* fn = pick(f64, log2Domain, mode, args.featureMode);
+  const void* fn = pick(f64, log2Domain, linear, mode, args.featureMode);
   if (ldsBytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(ldsBytes));
     if (e != hipSuccess) return e;

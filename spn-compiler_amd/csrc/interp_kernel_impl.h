@@ -120,6 +120,19 @@ __device__ __forceinline__ double rmax(double a, double b) { return __builtin_fm
 __device__ __forceinline__ float rfma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double rfma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
+// A Gaussian leaf from its three constants and the neutral element / combination of a product, in log space
+// (shift and den: den * ((x - mean)^2 + shift)) and in linear space (coef and den: coef * exp((x - mean)^2 * den)).
+template <bool LINEAR, typename R>
+__device__ __forceinline__ R gaussLeaf(R x, R mean, R c1, R c2) {
+  const R d = x - mean;
+  if constexpr (LINEAR) return c1 * ::exp(d * d * c2);
+  else return rfma(d, d, c1) * c2;
+}
+template <bool LINEAR, typename R>
+__device__ __forceinline__ R productStart() { return LINEAR ? R(1) : R(0); }
+template <bool LINEAR, typename R>
+__device__ __forceinline__ R productJoin(R acc, R v) { return LINEAR ? acc * v : acc + v; }
+
 // Constants are read at a signed offset from a pointer, not at an unsigned index into the
 // stream: only then may the compiler merge neighbouring reads into one wide scalar load.
 template <typename R>
@@ -227,11 +240,28 @@ struct Slots {
 // All instruction decoding goes through a pointer to the current instruction (`ip`) and signed
 // offsets from it, so that neighbouring words are fetched with wide scalar loads.
 
-template <typename R, bool LOG2, bool SPILL, int M>
+// LINEAR (here and below): the program computes with probabilities, not their logarithms (the reference's
+// computeInLogSpace=False, mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:242-304): products multiply, sums are plain
+// weighted sums, a Gaussian leaf is coef * exp((x - mean)^2 * den), and only the root takes a logarithm.
+template <typename R, bool LOG2, bool SPILL, int M, bool LINEAR = false>
 __device__ __forceinline__ code_ptr sumLayer(code_ptr ip, int k, const Slots<R, SPILL>& S) {
   typedef Math<R, LOG2> Mt;
   constexpr int RW = sizeof(R) / 4;
   code_ptr dsts = ip + 2, kids = dsts + M, w = kids + k;
+  if constexpr (LINEAR) {
+    R sum[M];
+#pragma unroll
+    for (int t = 0; t < M; ++t) sum[t] = R(0);
+#pragma unroll 4
+    for (int j = 0; j < k; ++j) {
+      const R x = S.rd(kids[j]);
+#pragma unroll
+      for (int t = 0; t < M; ++t) sum[t] = rfma(x, constAt<R>(w, (long(j) * M + t) * RW), sum[t]);
+    }
+#pragma unroll
+    for (int t = 0; t < M; ++t) S.wr(dsts[t], sum[t]);
+    return w + long(k) * M * RW;
+  }
   R m = R(-__builtin_huge_val());
 #pragma unroll 8
   for (int j = 0; j < k; ++j) m = rmax(m, S.rd(kids[j]));
@@ -252,11 +282,30 @@ __device__ __forceinline__ code_ptr sumLayer(code_ptr ip, int k, const Slots<R, 
 
 // M sums over the outer product of operand vectors a (NA slots) and b (NB slots):
 // out_j = ma + mb + log(sum_{r,c} w_j[r][c] * exp(a_r - ma) * exp(b_c - mb)), ma = max a, mb = max b.
-template <typename R, bool LOG2, bool SPILL, int M, int NB>
+template <typename R, bool LOG2, bool SPILL, int M, int NB, bool LINEAR = false>
 __device__ __forceinline__ code_ptr outerSum(code_ptr ip, int na, const Slots<R, SPILL>& S) {
   typedef Math<R, LOG2> Mt;
   constexpr int RW = sizeof(R) / 4;
   code_ptr dsts = ip + 2, as = dsts + M, bs = as + na, w = bs + NB;
+  if constexpr (LINEAR) {
+    R vb[NB], sum[M];
+#pragma unroll
+    for (int c = 0; c < NB; ++c) vb[c] = S.rd(bs[c]);
+#pragma unroll
+    for (int t = 0; t < M; ++t) sum[t] = R(0);
+    for (int r = 0; r < na; ++r) {
+      const R va = S.rd(as[r]);
+#pragma unroll
+      for (int c = 0; c < NB; ++c) {
+        const R e = va * vb[c];
+#pragma unroll
+        for (int t = 0; t < M; ++t) sum[t] = rfma(e, constAt<R>(w, ((long(r) * NB + c) * M + t) * RW), sum[t]);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < M; ++t) S.wr(dsts[t], sum[t]);
+    return w + long(na) * NB * M * RW;
+  }
   R eb[NB];
   R mb = R(-__builtin_huge_val());
 #pragma unroll
@@ -298,7 +347,7 @@ __device__ __forceinline__ code_ptr outerSum(code_ptr ip, int na, const Slots<R,
 struct __attribute__((packed, aligned(4))) StreamDouble {  // a double in the instruction stream: at a multiple of four bytes
   double value;
 };
-template <bool LOG2, bool SPILL, int NB>
+template <bool LOG2, bool SPILL, int NB, bool LINEAR = false>
 __device__ __forceinline__ code_ptr outerSumLaneWeights(code_ptr ip, int na, const StreamDouble* wGlobal, const Slots<double, SPILL>& S) {
   typedef Math<double, LOG2> Mt;
   constexpr int M = 8, V = NB / 2;  // vectors of sixteen weights per operand row
@@ -310,17 +359,20 @@ __device__ __forceinline__ code_ptr outerSumLaneWeights(code_ptr ip, int na, con
     eb[c] = S.rd(bs[c]);
     mb = rmax(mb, eb[c]);
   }
-  mb = rmax(mb, Mt::lowest());
+  mb = LINEAR ? 0.0 : rmax(mb, Mt::lowest());
   const StreamDouble* wl = wGlobal + (threadIdx.x & 15u);
   double W[2][V];
 #pragma unroll
   for (int v = 0; v < V; ++v) W[0][v] = wl[v * 16].value;
+  double ma = 0.0;
+  if constexpr (!LINEAR) {
 #pragma unroll
-  for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(eb[c] - mb);
-  double ma = -__builtin_huge_val();
+    for (int c = 0; c < NB; ++c) eb[c] = Mt::exp(eb[c] - mb);
+    ma = -__builtin_huge_val();
 #pragma unroll 8
-  for (int r = 0; r < na; ++r) ma = rmax(ma, S.rd(as[r]));
-  ma = rmax(ma, Mt::lowest());
+    for (int r = 0; r < na; ++r) ma = rmax(ma, S.rd(as[r]));
+    ma = rmax(ma, Mt::lowest());
+  }
   double acc[M];
 #pragma unroll
   for (int t = 0; t < M; ++t) acc[t] = 0.0;
@@ -332,7 +384,7 @@ __device__ __forceinline__ code_ptr outerSumLaneWeights(code_ptr ip, int na, con
       // the next row's weights (past the last row: the words that follow the instruction, read and not used)
 #pragma unroll
       for (int v = 0; v < V; ++v) W[half ^ 1][v] = wl[((row + 1) * V + v) * 16].value;
-      const double ea = Mt::exp(S.rd(as[row]) - ma);
+      const double ea = LINEAR ? S.rd(as[row]) : Mt::exp(S.rd(as[row]) - ma);
 #pragma unroll
       for (int c = 0; c < NB; ++c) {
         const double e = ea * eb[c];
@@ -363,7 +415,7 @@ __device__ __forceinline__ code_ptr outerSumLaneWeights(code_ptr ip, int na, con
   }
   const double base = ma + mb;
 #pragma unroll
-  for (int t = 0; t < M; ++t) S.wr(dsts[t], base + Mt::log(acc[t]));
+  for (int t = 0; t < M; ++t) S.wr(dsts[t], LINEAR ? acc[t] : base + Mt::log(acc[t]));
   return bs + NB + long(na) * NB * M * 2;
 }
 
@@ -580,12 +632,12 @@ __device__ __forceinline__ code_ptr outerSumMatrixAny(code_ptr ip, const Head& h
   return outerSumMatrix<LOG2, SPILL, TIERED, 8, 2>(ip, h, wGlobal, S);
 }
 
-template <typename R, bool LOG2, bool SPILL, int M>
+template <typename R, bool LOG2, bool SPILL, int M, bool LINEAR = false>
 __device__ __forceinline__ code_ptr outerSumNB(code_ptr ip, int na, int nb, const Slots<R, SPILL>& S) {
-  if (nb == 8) return outerSum<R, LOG2, SPILL, M, 8>(ip, na, S);
-  if (nb == 4) return outerSum<R, LOG2, SPILL, M, 4>(ip, na, S);
-  if (nb == 16) return outerSum<R, LOG2, SPILL, M, 16>(ip, na, S);
-  return outerSum<R, LOG2, SPILL, M, 2>(ip, na, S);
+  if (nb == 8) return outerSum<R, LOG2, SPILL, M, 8, LINEAR>(ip, na, S);
+  if (nb == 4) return outerSum<R, LOG2, SPILL, M, 4, LINEAR>(ip, na, S);
+  if (nb == 16) return outerSum<R, LOG2, SPILL, M, 16, LINEAR>(ip, na, S);
+  return outerSum<R, LOG2, SPILL, M, 2, LINEAR>(ip, na, S);
 }
 
 // The operand vectors of a leaf region: NA + NB products of G Gaussian leaves, the first NA over the features
@@ -845,7 +897,7 @@ __device__ __forceinline__ code_ptr leafInstruction(uint32_t op, code_ptr ip, co
 // n products of G Gaussian leaves each. The records are independent, so they are taken four at
 // a time: all constants of a group arrive in a few wide scalar loads and all feature reads of a
 // group are in flight together, instead of one dependent load chain per product.
-template <typename R, bool SPILL, int G, bool stagedMode, bool MARGINAL>
+template <typename R, bool SPILL, int G, bool stagedMode, bool MARGINAL, bool LINEAR = false>
 __device__ __forceinline__ code_ptr prodBatch(code_ptr ip, int n, const Slots<R, SPILL>& S, const InterpLaunch& a, unsigned long long row,
                                               bool useRegs, const FeatureRegs& regs) {
   constexpr int RW = sizeof(R) / 4, LEAF = 1 + 3 * RW, REC = 1 + G * LEAF, P = 4;
@@ -862,28 +914,26 @@ __device__ __forceinline__ code_ptr prodBatch(code_ptr ip, int n, const Slots<R,
       }
 #pragma unroll
     for (int q = 0; q < P; ++q) {
-      R acc = R(0);
+      R acc = productStart<LINEAR, R>();
 #pragma unroll
       for (int j = 0; j < G; ++j) {
         const long at = q * REC + 1 + j * LEAF + 1;
-        const R d = x[q][j] - constAt<R>(ip, at);
-        R v = rfma(d, d, constAt<R>(ip, at + RW)) * constAt<R>(ip, at + 2 * RW);
-        if (MARGINAL && a.marginal) v = (x[q][j] != x[q][j]) ? R(0) : v;
-        acc += v;
+        R v = gaussLeaf<LINEAR>(x[q][j], constAt<R>(ip, at), constAt<R>(ip, at + RW), constAt<R>(ip, at + 2 * RW));
+        if (MARGINAL && a.marginal) v = (x[q][j] != x[q][j]) ? productStart<LINEAR, R>() : v;
+        acc = productJoin<LINEAR>(acc, v);
       }
       S.wr(ip[q * REC], acc);
     }
   }
   for (; done < n; ++done, ip += REC) {
-    R acc = R(0);
+    R acc = productStart<LINEAR, R>();
 #pragma unroll
     for (int j = 0; j < G; ++j) {
       const uint32_t fw = ip[1 + j * LEAF];
       const R xv = stagedMode ? S.rd(fw) : (useRegs ? R(regs[fw % INTERP_FEATURE_REGISTERS]) : featureValue<R>(a.in, a.featureType, row + fw));
-      const R d = xv - constAt<R>(ip, 2 + j * LEAF);
-      R v = rfma(d, d, constAt<R>(ip, 2 + j * LEAF + RW)) * constAt<R>(ip, 2 + j * LEAF + 2 * RW);
-      if (MARGINAL && a.marginal) v = (xv != xv) ? R(0) : v;
-      acc += v;
+      R v = gaussLeaf<LINEAR>(xv, constAt<R>(ip, 2 + j * LEAF), constAt<R>(ip, 2 + j * LEAF + RW), constAt<R>(ip, 2 + j * LEAF + 2 * RW));
+      if (MARGINAL && a.marginal) v = (xv != xv) ? productStart<LINEAR, R>() : v;
+      acc = productJoin<LINEAR>(acc, v);
     }
     S.wr(ip[0], acc);
   }
@@ -956,7 +1006,7 @@ __device__ __forceinline__ code_ptr prodBatchTieredAny(code_ptr ip, int n, uint3
 }
 
 // Executes one instruction other than OP_END and returns the pointer to the next one.
-template <typename R, bool LOG2, bool SPILL, bool TIERED>
+template <typename R, bool LOG2, bool SPILL, bool TIERED, bool LINEAR>
 __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Slots<R, SPILL>& S, const InterpLaunch& a,
                                             const R* __restrict__ tables, unsigned long long row, bool stagedMode, code_ptr code0,
                                             const uint32_t* codeGlobal, bool useRegs, const FeatureRegs& regs) {
@@ -967,9 +1017,9 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
     const uint32_t dst = h.word(2);
     const int ns = int(h.word(3)), ng = int(h.word(4)), nt = int(h.word(5));
     ip += 5;
-    R acc = R(0);
+    R acc = productStart<LINEAR, R>();
 #pragma unroll 4
-    for (int j = 0; j < ns; ++j) acc += S.rd(ip[j]);
+    for (int j = 0; j < ns; ++j) acc = productJoin<LINEAR>(acc, S.rd(ip[j]));
     ip += ns;
 #pragma unroll 2
     for (int j = 0; j < ng; ++j) {
@@ -977,16 +1027,15 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
       const R mean = constAt<R>(ip, 1), shift = constAt<R>(ip, 1 + RW), den = constAt<R>(ip, 1 + 2 * RW);
       ip += 1 + 3 * RW;
       const R x = stagedMode ? S.rd(fw) : (useRegs ? R(regs[fw % INTERP_FEATURE_REGISTERS]) : featureValue<R>(a.in, a.featureType, row + fw));
-      const R d = x - mean;
-      R v = rfma(d, d, shift) * den;
-      if (a.marginal) v = (x != x) ? R(0) : v;
-      acc += v;
+      R v = gaussLeaf<LINEAR>(x, mean, shift, den);
+      if (a.marginal) v = (x != x) ? productStart<LINEAR, R>() : v;
+      acc = productJoin<LINEAR>(acc, v);
     }
     for (int j = 0; j < nt; ++j) {
       const uint32_t fw = ip[0], off = ip[1], L = ip[2];
       ip += 3;
       const uint32_t idx = stagedMode ? uint32_t(S.rd(fw)) : featureIndex(a.in, a.featureType, row + fw, L, a.marginal);
-      acc += tables[off + idx];
+      acc = productJoin<LINEAR>(acc, tables[off + idx]);
     }
     S.wr(dst, acc);
     return ip;
@@ -994,7 +1043,7 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
   if (op == OP_PRODBATCH) {
     const int n = int(w0 >> 8);
     const uint32_t flags = h.word(2), leaves = flags & 0xffu;
-    if constexpr (SPILL && TIERED) {
+    if constexpr (SPILL && TIERED && !LINEAR) {
       // Tier flags are valid (exactly the short pool is in LDS): no generic accesses unless a list is mixed.
       if (stagedMode && ((flags >> 8) & 3u) != 2u && ((flags >> 10) & 3u) != 2u && leaves != 3) {
         if (!a.marginal) {
@@ -1010,26 +1059,33 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
     // Staged features make the whole batch straight-line code; the direct form decides the input type per read.
     // Without marginal support (the common staged case) the NaN select is not compiled in at all.
     if (stagedMode && !a.marginal) {
-      if (leaves == 2) return prodBatch<R, SPILL, 2, true, false>(ip, n, S, a, row, useRegs, regs);
-      if (leaves == 1) return prodBatch<R, SPILL, 1, true, false>(ip, n, S, a, row, useRegs, regs);
-      if (leaves == 4) return prodBatch<R, SPILL, 4, true, false>(ip, n, S, a, row, useRegs, regs);
-      return prodBatch<R, SPILL, 3, true, false>(ip, n, S, a, row, useRegs, regs);
+      if (leaves == 2) return prodBatch<R, SPILL, 2, true, false, LINEAR>(ip, n, S, a, row, useRegs, regs);
+      if (leaves == 1) return prodBatch<R, SPILL, 1, true, false, LINEAR>(ip, n, S, a, row, useRegs, regs);
+      if (leaves == 4) return prodBatch<R, SPILL, 4, true, false, LINEAR>(ip, n, S, a, row, useRegs, regs);
+      return prodBatch<R, SPILL, 3, true, false, LINEAR>(ip, n, S, a, row, useRegs, regs);
     }
     if (stagedMode) {
-      if (leaves == 2) return prodBatch<R, SPILL, 2, true, true>(ip, n, S, a, row, useRegs, regs);
-      if (leaves == 1) return prodBatch<R, SPILL, 1, true, true>(ip, n, S, a, row, useRegs, regs);
-      if (leaves == 4) return prodBatch<R, SPILL, 4, true, true>(ip, n, S, a, row, useRegs, regs);
-      return prodBatch<R, SPILL, 3, true, true>(ip, n, S, a, row, useRegs, regs);
+      if (leaves == 2) return prodBatch<R, SPILL, 2, true, true, LINEAR>(ip, n, S, a, row, useRegs, regs);
+      if (leaves == 1) return prodBatch<R, SPILL, 1, true, true, LINEAR>(ip, n, S, a, row, useRegs, regs);
+      if (leaves == 4) return prodBatch<R, SPILL, 4, true, true, LINEAR>(ip, n, S, a, row, useRegs, regs);
+      return prodBatch<R, SPILL, 3, true, true, LINEAR>(ip, n, S, a, row, useRegs, regs);
     }
-    if (leaves == 2) return prodBatch<R, SPILL, 2, false, true>(ip, n, S, a, row, useRegs, regs);
-    if (leaves == 1) return prodBatch<R, SPILL, 1, false, true>(ip, n, S, a, row, useRegs, regs);
-    if (leaves == 4) return prodBatch<R, SPILL, 4, false, true>(ip, n, S, a, row, useRegs, regs);
-    return prodBatch<R, SPILL, 3, false, true>(ip, n, S, a, row, useRegs, regs);
+    if (leaves == 2) return prodBatch<R, SPILL, 2, false, true, LINEAR>(ip, n, S, a, row, useRegs, regs);
+    if (leaves == 1) return prodBatch<R, SPILL, 1, false, true, LINEAR>(ip, n, S, a, row, useRegs, regs);
+    if (leaves == 4) return prodBatch<R, SPILL, 4, false, true, LINEAR>(ip, n, S, a, row, useRegs, regs);
+    return prodBatch<R, SPILL, 3, false, true, LINEAR>(ip, n, S, a, row, useRegs, regs);
   }
   if (op == OP_SUM) {
     const int k = int(w0 >> 8);
     const uint32_t dst = h.word(2);
     ip += 2;
+    if constexpr (LINEAR) {
+      R sum = R(0);
+#pragma unroll 4
+      for (int j = 0; j < k; ++j) sum = rfma(S.rd(ip[long(j) * (1 + RW)]), constAt<R>(ip, long(j) * (1 + RW) + 1), sum);
+      S.wr(dst, sum);
+      return ip + long(k) * (1 + RW);
+    }
     if (k == 1) {
       S.wr(dst, S.rd(ip[0]) + constAt<R>(ip, 1));
       return ip + 1 + RW;
@@ -1068,12 +1124,12 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
   if (op == OP_SUMLAYER) {
     const int k = int(w0 >> 8);
     const uint32_t m = h.word(2);
-    if (m == 8) return sumLayer<R, LOG2, SPILL, 8>(ip, k, S);
-    if (m == 4) return sumLayer<R, LOG2, SPILL, 4>(ip, k, S);
-    return sumLayer<R, LOG2, SPILL, 2>(ip, k, S);
+    if (m == 8) return sumLayer<R, LOG2, SPILL, 8, LINEAR>(ip, k, S);
+    if (m == 4) return sumLayer<R, LOG2, SPILL, 4, LINEAR>(ip, k, S);
+    return sumLayer<R, LOG2, SPILL, 2, LINEAR>(ip, k, S);
   }
   const int na = int((w0 >> 8) & 0xffu), nb = int((w0 >> 16) & 0xffu);
-  if constexpr (sizeof(R) == 4) {
+  if constexpr (sizeof(R) == 4 && !LINEAR) {
     if (op == OP_LEAFQUADMM || op == OP_LEAFPAIRMM || op == OP_LEAFMM) {
       const FeatureSource fs{a.in, a.featureType, row};
       if (stagedMode) return leafInstruction<LOG2, SPILL, TIERED, true>(op, ip, h, na, nb, a.marginal != 0, code0, codeGlobal, fs, useRegs, regs, S);
@@ -1092,13 +1148,13 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
     // wavefront is at work here: idle lanes recompute the batch's last sample)
     if (m == 8 && (nb == 8 || nb == 4) && na % 2 == 0) {
       const StreamDouble* wGlobal = reinterpret_cast<const StreamDouble*>(codeGlobal + ((ip - code0) + 2 + 8 + na + nb));
-      if (nb == 8) return outerSumLaneWeights<LOG2, SPILL, 8>(ip, na, wGlobal, S);
-      return outerSumLaneWeights<LOG2, SPILL, 4>(ip, na, wGlobal, S);
+      if (nb == 8) return outerSumLaneWeights<LOG2, SPILL, 8, LINEAR>(ip, na, wGlobal, S);
+      return outerSumLaneWeights<LOG2, SPILL, 4, LINEAR>(ip, na, wGlobal, S);
     }
   }
-  if (m == 8) return outerSumNB<R, LOG2, SPILL, 8>(ip, na, nb, S);
-  if (m == 4) return outerSumNB<R, LOG2, SPILL, 4>(ip, na, nb, S);
-  return outerSumNB<R, LOG2, SPILL, 2>(ip, na, nb, S);
+  if (m == 8) return outerSumNB<R, LOG2, SPILL, 8, LINEAR>(ip, na, nb, S);
+  if (m == 4) return outerSumNB<R, LOG2, SPILL, 4, LINEAR>(ip, na, nb, S);
+  return outerSumNB<R, LOG2, SPILL, 2, LINEAR>(ip, na, nb, S);
 }
 
 // MODE 0: every slot lives in LDS. MODE 1: slots below ldsSlots (the program's short pool) live
@@ -1108,9 +1164,12 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
 // decided by the launch arguments (one kernel then carries both forms of every instruction that reads features);
 // 3: the program keeps its (at most 32) features in registers: they are read from the input row once per tile and the
 // feature fields of the instructions are register numbers, so no instruction fetches a feature from memory.
-template <typename R, bool LOG2, int MODE, int FEAT>
+template <typename R, bool LOG2, int MODE, int FEAT_OR_LINEAR>
 __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t* __restrict__ codeGlobal, InterpLaunch a) {
   typedef Math<R, LOG2> Mt;
+  // Flavour 4 is the linear-space one: feature mode decided at run time like flavour 2, values are probabilities.
+  constexpr bool LINEAR = FEAT_OR_LINEAR == 4;
+  constexpr int FEAT = LINEAR ? 2 : FEAT_OR_LINEAR;
   extern __shared__ __align__(16) unsigned char ldsRaw[];
   code_ptr code = (code_ptr)codeGlobal;
   const SPN_CONST uint32_t* staged = (const SPN_CONST uint32_t*)a.staged;
@@ -1173,12 +1232,12 @@ __global__ void __launch_bounds__(INTERP_BLOCK) spn_interp_kernel(const uint32_t
       }
       code_ptr next = ip + 1 + h.word(0);
       const Head hn = loadHead(codeGlobal, next - code);  // in flight while this instruction executes
-      if (MODE != 0 && spillPath) execute<R, LOG2, true, MODE == 1>(ip + 1, h, Sg, a, tables, row, stagedMode, code, codeGlobal, useRegs, regs);
-      else execute<R, LOG2, false, false>(ip + 1, h, Sl, a, tables, row, stagedMode, code, codeGlobal, useRegs, regs);
+      if (MODE != 0 && spillPath) execute<R, LOG2, true, MODE == 1, LINEAR>(ip + 1, h, Sg, a, tables, row, stagedMode, code, codeGlobal, useRegs, regs);
+      else execute<R, LOG2, false, false, LINEAR>(ip + 1, h, Sl, a, tables, row, stagedMode, code, codeGlobal, useRegs, regs);
       ip = next;
       h = hn;
     }
-    if (valid) out[i] = Mt::finish(result);
+    if (valid) out[i] = LINEAR ? R(::log(double(result))) : Mt::finish(result);
   }
 }
 

@@ -297,10 +297,13 @@ void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures) {
 
 namespace {
 InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t longRange, bool stagedLong) {
-  if (!o.useLogSpace) throw std::runtime_error("The interpreter kernel supports log-space computation only");
   InterpProgram p;
-  p.f64 = o.computeType == ComputeType::F64;
-  p.log2Domain = o.log2Domain;
+  // Linear space: probabilities in double, as the reference computes them (computeInLogSpace=False); the same
+  // instructions with other constants (linear weights everywhere, linear table values, Gaussian leaves as coefficient
+  // and natural-log exponent factor) and no matrix or scaled-vector forms.
+  p.linear = !o.useLogSpace;
+  p.f64 = p.linear || o.computeType == ComputeType::F64;
+  p.log2Domain = !p.linear && o.log2Domain;
   Builder b(g, p);
   const size_t N = g.nodes.size();
   auto isLeaf = [&](uint32_t i) { return g.nodes[i].kind != NodeKind::Product && g.nodes[i].kind != NodeKind::Sum; };
@@ -322,8 +325,11 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
     const auto& n = g.nodes[i];
     uint32_t L = featTableLen[n.feature];
     tableOffset[i] = uint32_t(p.tables.size());
-    for (uint32_t j = 0; j <= L; ++j) p.tables.push_back(b.logConst(j < n.table.size() ? n.table[j] : 0.0));
-    p.tables.push_back(0.0);
+    for (uint32_t j = 0; j <= L; ++j) {
+      const double pr = j < n.table.size() ? n.table[j] : 0.0;  // entry L: impossible
+      p.tables.push_back(p.linear ? pr : b.logConst(pr));
+    }
+    p.tables.push_back(p.linear ? 1.0 : 0.0);  // entry L + 1: the marginal value
   }
   uint32_t stagedSlots = 0;
   for (uint32_t f = 0; f < g.numFeatures; ++f) {
@@ -716,8 +722,13 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       else if (p.featureMode == FEAT_REGISTER) b.word(valueSlotOf[leaf.feature]);
       else b.word(leaf.feature);
       b.real(leaf.mean);
-      b.real(coef / den);  // value = den * (d * d + coef / den): one multiply-add and one multiply, each with one constant
-      b.real(den * b.scale);
+      if (p.linear) {
+        b.real(std::exp(coef));  // value = coef * exp(d * d * den)
+        b.real(den);
+      } else {
+        b.real(coef / den);  // value = den * (d * d + coef / den): one multiply-add and one multiply, each with one constant
+        b.real(den * b.scale);
+      }
     } else {
       if (p.featureMode == FEAT_STAGED) slotWord(indexSlotOf[leaf.feature]);
       else b.word(leaf.feature);
@@ -847,7 +858,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
         slotWord(slotOf[in.node]);
         for (uint32_t j = 0; j < cnt; ++j) {
           slotWord(slotOf[n.children[j]]);
-          if (cnt == 1) b.real(b.logConst(n.weights[j]));  // single child: value + log weight
+          if (cnt == 1 && !p.linear) b.real(b.logConst(n.weights[j]));  // single child: value + log weight
           else b.real(n.weights[j]);
         }
         b.end(at);
@@ -1053,7 +1064,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
   std::ostringstream hdr;
   hdr << "; interpreter program for SPN '" << g.name << "': " << instrs.size() << " instructions, " << p.code.size() << " words, "
       << p.numSlots << " value slots (" << p.reservedSlots << " staged features, " << (p.numSlots - p.shortSlots) << " long-lived), compute " << (p.f64 ? "f64" : "f32")
-      << (p.log2Domain ? " log2-domain" : "") << ", features " << (p.featureMode == FEAT_STAGED ? "staged" : (p.featureMode == FEAT_REGISTER ? "in registers" : "direct")) << "\n";
+      << (p.log2Domain ? " log2-domain" : "") << (p.linear ? " linear space" : "") << ", features " << (p.featureMode == FEAT_STAGED ? "staged" : (p.featureMode == FEAT_REGISTER ? "in registers" : "direct")) << "\n";
   p.listing = hdr.str() + b.txt.str();
   return p;
 }

@@ -72,6 +72,7 @@ struct StagedFeature {
 struct InterpProgram {
   bool f64 = false;
   bool log2Domain = true;
+  bool linear = false;                 // values are probabilities, not logarithms (the reference's computeInLogSpace=False); always f64
   FeatureMode featureMode = FEAT_STAGED;
   std::vector<uint32_t> code;
   std::vector<double> tables;          // pool of leaf tables in the kernel's log domain

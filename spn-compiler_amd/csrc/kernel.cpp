@@ -80,7 +80,7 @@ uint32_t spilledRegisters(const std::vector<char>& code) {
 }
 
 // ---- kernel file: magic, then tagged little-endian fields ----
-const char kMagic[8] = {'S', 'P', 'N', 'C', 'H', 'I', 'P', 3};
+const char kMagic[8] = {'S', 'P', 'N', 'C', 'H', 'I', 'P', 4};
 
 struct Writer {
   std::vector<char> buf;
@@ -279,11 +279,10 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
   // (mlir/lib/Dialect/LoSPN/Passes/LoSPNTaskPartitioner.cpp:36-148); the straight-line kernels are cut the same way
   // (partition.cpp). The interpreter's code does not grow with the graph and ignores the option.
   const uint64_t jitLimit = uint64_t(std::max(0, o.jitMaxOps));
-  bool useInterp = o.kernelMode == KernelMode::Interpreter || (o.kernelMode == KernelMode::Auto && ops > jitLimit);
-  if (useInterp && !o.useLogSpace) {
-    if (o.kernelMode == KernelMode::Interpreter) fatal("COMPILATION ERROR: the interpreter kernel supports log-space computation only");
-    useInterp = false;
-  }
+  // In linear space (computed in double, as in the reference) the interpreter takes what is too large for one
+  // straight-line kernel as well, unless the caller asked for tasks: its program is there at once, where the kernels
+  // of a graph cut into tasks take hipRTC minutes (47 k nodes: 100-125 s).
+  bool useInterp = o.kernelMode == KernelMode::Interpreter || (o.kernelMode == KernelMode::Auto && ops > jitLimit && (o.useLogSpace || o.maxTaskSize <= 0));
   if (useInterp) {
     k->kind_ = SPNC_HIP_KERNEL_INTERPRETER;
     k->prog_ = buildInterpProgram(g, o);
@@ -295,11 +294,7 @@ std::unique_ptr<Kernel> Kernel::compile(const std::string& queryPath, const std:
   } else {
     k->kind_ = SPNC_HIP_KERNEL_JIT;
     TaskPlan plan;
-    // Without "maxTaskSize", a graph that is larger than what one straight-line kernel is built for (it is here because
-    // linear-space computation or the caller ruled the interpreter out) is cut into tasks of 2000 operations: hipRTC
-    // time then grows with the graph instead of with its square, and no kernel outgrows the register file.
     int taskSize = o.maxTaskSize;
-    if (taskSize <= 0 && ops > jitLimit && o.kernelMode != KernelMode::Jit) taskSize = 2000;
     if (taskSize > 0) plan = partitionGraph(g, taskSize);
     JitSource js;
     if (plan.tasks.size() > 1) {
@@ -418,6 +413,7 @@ void Kernel::save(const std::string& path) const {
   } else {
     w.u32(prog_.f64);
     w.u32(prog_.log2Domain);
+    w.u32(prog_.linear);
     w.u32(prog_.featureMode);
     w.vec(prog_.code);
     w.vec(prog_.tables);
@@ -484,6 +480,7 @@ std::unique_ptr<Kernel> Kernel::load(const std::string& kernelFile) {
   } else if (k->kind_ == SPNC_HIP_KERNEL_INTERPRETER) {
     k->prog_.f64 = r.u32() != 0;
     k->prog_.log2Domain = r.u32() != 0;
+    k->prog_.linear = r.u32() != 0;
     k->prog_.featureMode = FeatureMode(r.u32());
     k->prog_.code = r.vec<uint32_t>();
     k->prog_.tables = r.vec<double>();
@@ -602,7 +599,7 @@ void Kernel::queryDevice() {
     // The kernel's own static LDS (the float64 log2 flavour keeps 4.7 KiB of exp2/log2 tables there) comes out of
     // the same memory: without it in the sum a program of 40 slots would leave room for one block per CU, not two.
     size_t maxBlock = 0, staticLds = 0;
-    hipCheck(interpreterMaxLds(prog_.f64, prog_.log2Domain, prog_.featureMode, &maxBlock, &staticLds), "LDS limit query");
+    hipCheck(interpreterMaxLds(prog_.f64, prog_.log2Domain, prog_.linear, prog_.featureMode, &maxBlock, &staticLds), "LDS limit query");
     size_t budget = std::min<size_t>(maxBlock, size_t(ldsPerCU) / 2);
     budget = budget > staticLds ? budget - staticLds : 0;
     uint32_t cap = uint32_t(budget / (INTERP_BLOCK * rb));
@@ -619,7 +616,7 @@ void Kernel::queryDevice() {
     }
     ldsBytes_ = size_t(ldsSlots_) * INTERP_BLOCK * rb;
     int nb = 0;
-    hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, interpMode_, prog_.featureMode, ldsBytes_, &nb), "occupancy query");
+    hipCheck(interpreterOccupancy(prog_.f64, prog_.log2Domain, prog_.linear, interpMode_, prog_.featureMode, ldsBytes_, &nb), "occupancy query");
     blocksPerCU_ = std::max(1, nb);
     if (gridPolicy_ > 0) blocksPerCU_ = std::min(blocksPerCU_, gridPolicy_);  // "hip-blocks-per-cu": fewer than fit
   }
@@ -820,7 +817,7 @@ void Kernel::launchProgram(size_t n, const void* dIn, void* dOut, const uint32_t
   a.spillSlots = prog_.numSlots - ldsSlots_;
   a.marginal = marginal_ ? 1u : 0u;
   a.mathTables = prog_.mathTables;
-  hipCheck(launchInterpreter(a, prog_.f64, prog_.log2Domain, interpMode_, grid, ldsBytes_, stream), "interpreter launch");
+  hipCheck(launchInterpreter(a, prog_.f64, prog_.log2Domain, prog_.linear, interpMode_, grid, ldsBytes_, stream), "interpreter launch");
 }
 
 void Kernel::executeDevice(size_t n, const void* dIn, void* dOut, hipStream_t stream) {

@@ -122,8 +122,9 @@ def test_golden_outputs_f32(native, tmp_path, name, variant):
 
 @pytest.mark.parametrize("opts", [{"hip-compute-type": "float64"}, {"hip-compute-type": "float64", "hip-sum-form": "pairwise"},
                                   {"hip-compute-type": "float64", "hip-kernel": "interpreter"},
-                                  {"hip-compute-type": "float64", "hip-kernel": "interpreter", "hip-log2-domain": "false"}, {"use-log-space": "false"}],
-                         ids=["log-f64", "log-f64-pairwise", "log-f64-interp", "log-f64-interp-natural", "linear-f64"])
+                                  {"hip-compute-type": "float64", "hip-kernel": "interpreter", "hip-log2-domain": "false"}, {"use-log-space": "false"},
+                                  {"use-log-space": "false", "hip-kernel": "interpreter"}, {"use-log-space": "false", "hip-kernel": "jit", "maxTaskSize": 2000}],
+                         ids=["log-f64", "log-f64-pairwise", "log-f64-interp", "log-f64-interp-natural", "linear-f64", "linear-f64-interp", "linear-f64-tasks"])
 @pytest.mark.parametrize("name", ["NIPS5", "nltcs", "plants"])
 def test_golden_outputs_f64(native, tmp_path, name, opts):
     if name == "nltcs" and "hip-sum-form" in opts:
@@ -136,8 +137,11 @@ def test_golden_outputs_f64(native, tmp_path, name, opts):
         path = model_as_query(os.path.join(GOLDEN, name + ".bin"), "float64", str(tmp_path / "q.bin"))
     k = compile_query(native, path, **opts)
     if name == "nltcs" and "use-log-space" in opts:
-        # linear space rules the interpreter out; a graph this size is cut into tasks without being asked
-        assert k.info()["kernel_kind"] == 1 and k.info()["num_tasks"] > 1
+        # a graph this size in linear space: the interpreter unless the caller asks for straight-line kernels, then cut into tasks
+        if opts.get("hip-kernel") == "jit":
+            assert k.info()["kernel_kind"] == 1 and k.info()["num_tasks"] > 1
+        else:
+            assert k.info()["kernel_kind"] == 2
     got = run(k, X)
     assert got.dtype == np.float64
     assert np.abs(got - ref).max() <= F64_TOL
@@ -300,6 +304,42 @@ def test_reference_queries_without_expected_outputs(native, name, opts):
         assert np.abs(got - want).max() <= (1e-9 if "use-log-space" in opts else F64_TOL)
     else:
         assert within_f32(got, want), np.abs(got - want).max()
+
+
+def test_the_47k_node_model_in_linear_space(native, tmp_path):
+    """fashion_mnist.bin computed with probabilities instead of logarithms (the reference's computeInLogSpace=False, which
+    yields float64): the interpreter takes it, so compiling is a matter of a second. The product of 784 densities leaves
+    the double range (log-likelihoods near -1000 even at the leaves' means), where the reference's arithmetic ends in
+    log(0) = -inf as well: that is what the oracle's restatement of the reference's linear kernel gives for every row."""
+    import time
+    path = model_as_query(os.path.join(GOLDEN, "fashion_mnist.bin"), "float64", str(tmp_path / "q.bin"))
+    m = sm.load_model(path)
+    X = np.random.default_rng(12).random((200, 784))
+    t0 = time.time()
+    k = compile_query(native, path, **{"use-log-space": "false"})
+    assert time.time() - t0 < 10 and k.info()["kernel_kind"] == 2 and k.info()["dtype"] == "float64"
+    got = run(k, X)
+    want = ev.ll_linear_f64(m, X, marginal=False)
+    assert got.dtype == np.float64 and np.array_equal(np.isneginf(got), np.isneginf(want)) and not np.isnan(got).any()
+
+
+@pytest.mark.parametrize("cfg", ["c2", "c3", "c4", "c5"])
+def test_benchmark_configurations_in_linear_space_on_the_interpreter(native, cfg):
+    """Linear space (probabilities, float64) on the interpreter against the oracle's restatement of the reference's linear
+    kernel (mlir/lib/Conversion/LoSPNtoCPU/NodePatterns.cpp:242-304): Gaussian and table leaves, missing features, sums
+    over outer products, the region graph that the interpreter takes by itself."""
+    from spnc import synthetic as syn
+    c = syn.CONFIGS[cfg]
+    spn, X = c["spn"](), c["inputs"](1500)
+    opts = {"use-log-space": "false"} if cfg == "c4" else {"use-log-space": "false", "hip-kernel": "interpreter"}
+    k = compile_spn(native, spn, c["dtype"], marginal=c["marginal"], **opts)
+    assert k.info()["kernel_kind"] == 2 and "linear space" in k.source()
+    got = run(k, X)
+    want = ev.ll_linear_f64(oracle_model(spn, c["dtype"]), X, marginal=c["marginal"])
+    finite = np.isfinite(want)
+    assert got.dtype == np.float64 and finite.sum() > 1000
+    assert np.array_equal(np.isneginf(got), np.isneginf(want))
+    assert np.abs(got[finite] - want[finite]).max() <= F64_TOL
 
 
 @pytest.mark.parametrize("opts", [{}, {"hip-compute-type": "float64"}, {"hip-log2-domain": "false"}], ids=["f32", "f64", "f32-natural"])
