@@ -643,25 +643,26 @@ __device__ __forceinline__ code_ptr outerSumNB(code_ptr ip, int na, int nb, cons
 // The operand vectors of a leaf region: NA + NB products of G Gaussian leaves, the first NA over the features
 // x[0..G), the others over x[G..2G); constants (mean, shift, den per leaf) at ip[rec...]. Returns exp2(product -
 // max) per list in ea / eb and the sum of the two maxima.
-template <bool LOG2, int NA, int NB, int G, bool MARGINAL>
-__device__ __forceinline__ float leafOperands(code_ptr ip, long rec, const float* x, float* ea, float* eb) {
-  typedef Math<float, LOG2> Mt;
-  float e[NA + NB];
+template <bool LOG2, int NA, int NB, int G, bool MARGINAL, typename R = float>
+__device__ __forceinline__ R leafOperands(code_ptr ip, long rec, const R* x, R* ea, R* eb) {
+  typedef Math<R, LOG2> Mt;
+  constexpr int RW = sizeof(R) / 4;
+  R e[NA + NB];
 #pragma unroll
   for (int i = 0; i < NA + NB; ++i) {
-    float acc = 0.f;
+    R acc = R(0);
 #pragma unroll
     for (int j = 0; j < G; ++j) {
-      const long at = rec + (i * G + j) * 3;
-      const float xv = x[(i < NA ? 0 : G) + j];
-      const float d = xv - constAt<float>(ip, at);
-      float v = rfma(d, d, constAt<float>(ip, at + 1)) * constAt<float>(ip, at + 2);
-      if (MARGINAL) v = (xv != xv) ? 0.f : v;
+      const long at = rec + (i * G + j) * 3 * RW;
+      const R xv = x[(i < NA ? 0 : G) + j];
+      const R d = xv - constAt<R>(ip, at);
+      R v = rfma(d, d, constAt<R>(ip, at + RW)) * constAt<R>(ip, at + 2 * RW);
+      if (MARGINAL) v = (xv != xv) ? R(0) : v;
       acc += v;
     }
     e[i] = acc;
   }
-  float ma = -__builtin_huge_valf(), mb = -__builtin_huge_valf();
+  R ma = R(-__builtin_huge_val()), mb = R(-__builtin_huge_val());
 #pragma unroll
   for (int r = 0; r < NA; ++r) ma = rmax(ma, e[r]);
 #pragma unroll
@@ -861,6 +862,145 @@ __device__ __forceinline__ code_ptr leafQuadMatrix(code_ptr ip, const Head& h, c
   }
   matrixChainAndStore<LOG2, SPILL, 8, 8>(pv[0], pv[1], ATOP, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
   return ip + 2 + M + 1 + 8 * G + 4 * RECS + 2 * PAIRW + 64 * M;
+}
+
+// ---- The fused leaf instructions in double precision ----
+// No matrix instruction helps here (the double ones run at the rate of the vector unit and want four samples per group
+// of lanes); what the matrix form buys the float kernels, weights that reach the arithmetic without scalar loads and
+// scalar operands, the double kernels get from the cross-lane operand of v_fmac_f64 (outerSumLaneWeights above): the
+// weights lie product-major in the stream, eight sums per product, so a register pair loaded with sixteen consecutive
+// weights serves the eight sums of two products. Result vectors inside an instruction stay linear and unscaled, as in the
+// float forms; an instruction's own result is written as log2 values (doubles have the range for the products of a
+// whole instruction, and the consumer is an ordinary outer sum).
+
+// The sixteen multiply-adds of one lane vector: the eight sums of two products.
+__device__ __forceinline__ void laneVector(double* acc, double w, double e0, double e1) {
+  asm("v_fmac_f64_dpp %0, %8, %9 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %1, %8, %9 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %2, %8, %9 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %3, %8, %9 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %4, %8, %9 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %5, %8, %9 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %6, %8, %9 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %7, %8, %9 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %0, %8, %10 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %1, %8, %10 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %2, %8, %10 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %3, %8, %10 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %4, %8, %10 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %5, %8, %10 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %6, %8, %10 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f64_dpp %7, %8, %10 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+      : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+      : "v"(w), "v"(e0), "v"(e1));
+}
+
+// acc[t] = sum over products k = r NB + c of w[k][t] ea[r] eb[c]. A loop over the operand rows, two per round with the
+// vectors of the row after next requested meanwhile: unrolled over all products the chain of an 8x8 sum alone is 4.6 KiB of
+// instructions that every wavefront would stream through the instruction cache once per use.
+template <int NA, int NB>
+__device__ __forceinline__ void laneChain(const double* ea, const double* eb, const StreamDouble* wGlobal, double* acc) {
+  constexpr int V = NB / 2;  // vectors of sixteen weights per operand row
+  static_assert(NA % 2 == 0, "operand rows are taken two at a time");
+  const StreamDouble* wl = wGlobal + (threadIdx.x & 15u);
+  double W[2][V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) W[0][v] = wl[v * 16].value;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) acc[t] = 0.0;
+  SPN_PRIO_CHAIN();
+#pragma unroll 1
+  for (int r = 0; r < NA; r += 2) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int row = r + half;
+      // the next row's weights (past the last row: the words that follow, read and not used)
+#pragma unroll
+      for (int v = 0; v < V; ++v) W[half ^ 1][v] = wl[((row + 1) * V + v) * 16].value;
+      const double ear = ea[row];
+#pragma unroll
+      for (int v = 0; v < V; ++v) laneVector(acc, W[half][v], ear * eb[2 * v], ear * eb[2 * v + 1]);
+    }
+  }
+  SPN_PRIO_LATENCY();
+}
+
+// One leaf region of N x N products of G Gaussian leaves: its eight sums, linear and unscaled, in v; returns the sum of the
+// two operand maxima (log2). rec: offset of its constants from ip (in words), w: its weights.
+template <bool LOG2, int N, int G, bool MARGINAL>
+__device__ __forceinline__ double leafRegionLanes(code_ptr ip, long rec, const double* x, const StreamDouble* w, double* v) {
+  double ea[N], eb[N];
+  const double base = leafOperands<LOG2, N, N, G, MARGINAL, double>(ip, rec, x, ea, eb);
+  laneChain<N, N>(ea, eb, w, v);
+  return base;
+}
+
+template <int COUNT, bool SPILL>
+__device__ __forceinline__ void readLeafFeaturesDouble(const Slots<double, SPILL>& S, const Head& h, int pos, bool staged, const FeatureSource& fs, double* x) {
+  if (staged) {
+#pragma unroll
+    for (int j = 0; j < COUNT; ++j) x[j] = S.rd(h.word(pos + j));
+  } else {
+#pragma unroll
+    for (int j = 0; j < COUNT; ++j) x[j] = featureValue<double>(fs.in, fs.type, fs.row + h.word(pos + j));
+  }
+}
+
+template <bool LOG2, bool SPILL>
+__device__ __forceinline__ void storeLogVector(const Slots<double, SPILL>& S, const Head& h, int dstPos, double base, const double* acc) {
+  typedef Math<double, LOG2> Mt;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) S.wr(h.word(dstPos + t), base + Mt::log(acc[t]));
+}
+
+// OP_LEAFMM, OP_LEAFPAIRMM and OP_LEAFQUADMM of a double program: REGIONS = 1, 2 or 4 leaf regions of N x N products.
+// Words: opcode, format, eight destinations, a scale field (unused), 2 G feature fields per region, the regions'
+// constants, then the weights (product-major): one region: its own; a pair: region, region, the 8x8 sum over them;
+// a quad: pair, pair, the 8x8 sum over the pairs.
+template <bool LOG2, bool SPILL, int REGIONS, int N, int G, bool MARGINAL>
+__device__ __forceinline__ code_ptr leafLanes(code_ptr ip, const Head& h, const uint32_t* words, bool staged, const FeatureSource& fs,
+                                               const Slots<double, SPILL>& S) {
+  constexpr int M = 8, DST = 3, FEAT = DST + M + 1, NF = 2 * G * REGIONS, REC = FEAT + NF - 1;  // REC: offset of the constants from ip
+  constexpr int RECW = 2 * N * G * 3 * 2;                          // words of one region's constants
+  constexpr int LEAFW = N * N * M, TOPW = 64 * M, PAIRW = 2 * LEAFW + TOPW;  // weights (doubles) of a region, an 8x8 sum, a pair
+  const StreamDouble* w = reinterpret_cast<const StreamDouble*>(words + REC + REGIONS * RECW);  // `words`: ip's word in global memory
+  double x[NF];
+  readLeafFeaturesDouble<NF>(S, h, FEAT, staged, fs, x);
+  double out[M], base = 0.0;
+  if constexpr (REGIONS == 1) {
+    base = leafRegionLanes<LOG2, N, G, MARGINAL>(ip, REC, x, w, out);
+  } else if constexpr (REGIONS == 2) {
+    double va[M], vb[M];
+    base = leafRegionLanes<LOG2, N, G, MARGINAL>(ip, REC, x, w, va);
+    base += leafRegionLanes<LOG2, N, G, MARGINAL>(ip, REC + RECW, x + 2 * G, w + LEAFW, vb);
+    laneChain<8, 8>(va, vb, w + 2 * LEAFW, out);
+  } else {
+    double pv[2][M];
+#pragma unroll
+    for (int pair = 0; pair < 2; ++pair) {
+      double va[M], vb[M];
+      base += leafRegionLanes<LOG2, N, G, MARGINAL>(ip, REC + (2 * pair) * RECW, x + (2 * pair) * 2 * G, w + pair * PAIRW, va);
+      base += leafRegionLanes<LOG2, N, G, MARGINAL>(ip, REC + (2 * pair + 1) * RECW, x + (2 * pair + 1) * 2 * G, w + pair * PAIRW + LEAFW, vb);
+      laneChain<8, 8>(va, vb, w + pair * PAIRW + 2 * LEAFW, pv[pair]);
+    }
+    laneChain<8, 8>(pv[0], pv[1], w + 2 * PAIRW, out);
+  }
+  storeLogVector<LOG2>(S, h, DST, base, out);
+  constexpr int WEIGHTS = REGIONS == 1 ? LEAFW : (REGIONS == 2 ? PAIRW : 2 * PAIRW + TOPW);
+  return ip + REC + REGIONS * RECW + WEIGHTS * 2;
+}
+
+template <bool LOG2, bool SPILL, int REGIONS, int N>
+__device__ __forceinline__ code_ptr leafLanesG(code_ptr ip, const Head& h, uint32_t leaves, bool marginal, const uint32_t* stream, bool staged,
+                                                const FeatureSource& fs, const Slots<double, SPILL>& S) {
+  if (!marginal) {
+    if (leaves == 2) return leafLanes<LOG2, SPILL, REGIONS, N, 2, false>(ip, h, stream, staged, fs, S);
+    if (leaves == 1 || REGIONS == 4) return leafLanes<LOG2, SPILL, REGIONS, N, 1, false>(ip, h, stream, staged, fs, S);
+    return leafLanes<LOG2, SPILL, REGIONS, N, REGIONS == 4 ? 1 : 4, false>(ip, h, stream, staged, fs, S);
+  }
+  if (leaves == 2) return leafLanes<LOG2, SPILL, REGIONS, N, 2, true>(ip, h, stream, staged, fs, S);
+  if (leaves == 1 || REGIONS == 4) return leafLanes<LOG2, SPILL, REGIONS, N, 1, true>(ip, h, stream, staged, fs, S);
+  return leafLanes<LOG2, SPILL, REGIONS, N, REGIONS == 4 ? 1 : 4, true>(ip, h, stream, staged, fs, S);
 }
 
 // The three fused leaf instructions. STAGED: their feature fields are slots of staged values, else input columns.
@@ -1139,6 +1279,18 @@ __device__ __forceinline__ code_ptr execute(code_ptr ip, const Head& h, const Sl
       // The weights start after the two header words, eight destinations, na + nb operands and three scale slots.
       const float* wGlobal = reinterpret_cast<const float*>(codeGlobal) + ((ip - code0) + 13 + na + nb);
       return outerSumMatrixAny<LOG2, SPILL, TIERED>(ip, h, na, nb, wGlobal, S);
+    }
+  }
+  if constexpr (sizeof(R) == 8 && !LINEAR) {
+    if (op == OP_LEAFQUADMM || op == OP_LEAFPAIRMM || op == OP_LEAFMM) {
+      const FeatureSource fs{a.in, a.featureType, row};
+      const uint32_t leaves = (h.word(2) >> 12) & 0xfu;
+      const uint32_t* stream = codeGlobal + (ip - code0);  // this instruction's words in global memory
+      const bool marginal = a.marginal != 0;
+      if (op == OP_LEAFQUADMM) return leafLanesG<LOG2, SPILL, 4, 4>(ip, h, leaves, marginal, stream, stagedMode, fs, S);
+      if (op == OP_LEAFPAIRMM) return leafLanesG<LOG2, SPILL, 2, 4>(ip, h, leaves, marginal, stream, stagedMode, fs, S);
+      if (na == 4) return leafLanesG<LOG2, SPILL, 1, 4>(ip, h, leaves, marginal, stream, stagedMode, fs, S);
+      return leafLanesG<LOG2, SPILL, 1, 8>(ip, h, leaves, marginal, stream, stagedMode, fs, S);
     }
   }
   // OP_OUTERSUM

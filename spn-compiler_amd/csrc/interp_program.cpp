@@ -270,7 +270,9 @@ void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures) {
       case OP_LEAFPAIRMM:
       case OP_LEAFQUADMM: {
         const uint32_t na = (w0 >> 8) & 0xffu, nb = (w0 >> 16) & 0xffu, G = (w1 >> 12) & 0xfu, featTier = (w1 >> 16) & 3u;
-        if (p.f64 || (w1 & 0xffu) != 8) bad("leaf region shape", pc);
+        if (p.linear || (w1 & 0xffu) != 8) bad("leaf region shape", pc);
+        const size_t rw = p.f64 ? 2 : 1;  // words per constant and per weight
+        if (p.f64 && ((w1 >> 8) & 1u)) bad("scaled result in a double program", pc);
         size_t regions, products, weights;
         if (op == OP_LEAFMM) {
           if (!((na == 4 && nb == 4) || (na == 8 && nb == 8)) || !(G == 1 || G == 2 || G == 4)) bad("leaf region shape", pc);
@@ -282,7 +284,7 @@ void checkInterpProgram(const InterpProgram& p, uint32_t numFeatures) {
           if (na != 4 || nb != 0 || !(G == 1 || G == 2)) bad("leaf region quad shape", pc);
           regions = 4, products = 32, weights = 2 * (2 * 128 + 512) + 512;
         }
-        need(2 + 8 + 1 + 2 * regions * G + products * G * 3 + weights);
+        need(2 + 8 + 1 + 2 * regions * G + (products * G * 3 + weights) * rw);
         list(first + 2, 8, (w0 >> 28) & 3u, (w1 >> 11) & 1u);
         if ((w1 >> 8) & 1u) slot(first + 10);
         for (size_t j = 0; j < 2 * regions * G; ++j) feature(first + 11 + j, staged ? featTier : 2);
@@ -508,7 +510,9 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
       const Instr& in = instrs[k];
       if (in.op != OP_OUTERSUM) continue;
       const Outer& outer = outerOf.at(g.nodes[in.node].children);
-      matrixInstr[k] = !p.f64 && in.defs.size() == 8 && o.interpMatrixCore &&
+      // (double programs: the same instructions qualify, as candidates for the fused leaf forms, whose weights go
+      // through lanes; on their own they stay ordinary outer sums and no vector between them is scaled)
+      matrixInstr[k] = !p.linear && in.defs.size() == 8 && o.interpMatrixCore &&
                        matrixFormShape(uint32_t(outer.a.size()), uint32_t(outer.b.size()));
     }
     std::vector<std::vector<uint32_t>> readers(N);
@@ -812,7 +816,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
           if (scaleSlotOfNode[s] != NONE && blockOfNode[s] < 0) releaseSlot(scaleSlotOfNode[s]);  // else part of the block
         }
     }
-    if (in.op == OP_OUTERSUM && matrixInstr[k] && o.interpVectorBlocks) {
+    if (in.op == OP_OUTERSUM && matrixInstr[k] && !p.f64 && o.interpVectorBlocks) {
       const uint32_t base = allocBlock(in.defs[0]);
       for (uint32_t t = 0; t < in.defs.size(); ++t) {
         slotOf[in.defs[t]] = base + t;
@@ -886,7 +890,7 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
         // A single leftover sum is encoded as a layer of two identical sums writing the same slot.
         std::vector<uint32_t> defs = in.defs;
         if (m == 1) defs.push_back(in.defs[0]);
-        const bool matrixForm = matrixInstr[k];
+        const bool matrixForm = matrixInstr[k] && !p.f64;  // double programs: the fused leaf forms below, else an ordinary outer sum
         const size_t at = b.begin();
         // Matrix form: bits 24-29 say where each slot list lives (0 all in the short pool, 1 all in the long pool,
         // 2 mixed), so the kernel picks the access instructions per list, not per slot; bits 30 and 31 say that
@@ -934,6 +938,11 @@ InterpProgram buildWithRange(const Graph& g, const CompileOptions& o, uint32_t l
               }
         };
         auto emitMatrixWeights = [&](const std::vector<uint32_t>& sums, uint32_t products) {
+          if (p.f64) {  // product-major, the eight sums of a product side by side: sixteen weights per lane vector
+            for (uint32_t q = 0; q < products; ++q)
+              for (uint32_t t = 0; t < 8; ++t) b.real(g.nodes[sums[t]].weights[q]);
+            return;
+          }
           for (uint32_t grp = 0; grp < products / 16; ++grp)
             for (uint32_t half = 0; half < 2; ++half)
               for (uint32_t lane = 0; lane < 64; ++lane) b.real(g.nodes[sums[half * 4 + lane % 4]].weights[grp * 16 + lane / 4]);

@@ -1001,6 +1001,29 @@ def test_quads_of_leaf_regions_inside_the_outer_sum(native, count, leaves, regio
         assert within_f32(got, want64), opts
 
 
+@pytest.mark.parametrize("count,leaves,regions,paired,want", [
+    (4, 2, 9, 2, (2, 0, 1)), (4, 1, 9, 2, (2, 0, 1)), (4, 4, 5, 2, (0, 2, 1)), (8, 2, 3, 0, (0, 0, 3)), (8, 4, 3, 0, (0, 0, 3)),
+    (4, 1, 5, 1, (0, 2, 1)), (4, 2, 13, 2, (3, 0, 1)),
+])
+@pytest.mark.parametrize("marginal", [False, True])
+def test_fused_leaf_instructions_in_float64(native, count, leaves, regions, paired, want, marginal):
+    """The instructions over one, two and four leaf regions in a double program: the weights reach the multiply-adds
+    through lanes (v_fmac_f64 with a cross-lane operand), the vectors inside an instruction stay linear, its result is
+    written as log2 values. Against the closed form to 1e-10, with the slots in either tier and with staged features."""
+    spn, X = _leaf_region_graph(1700 + 10 * count + leaves + regions, count, leaves, regions, marginal, paired=paired)
+    want64 = ev.ll_closed_f64(oracle_model(spn, "float64"), X, marginal=marginal)
+    for opts in ({}, {"hip-interp-lds-slots": 6}, {"hip-interp-staged-features": "spill"}, {"hip-interp-staged-features": "lds", "hip-interp-lds-slots": 40},
+                 {"hip-interp-leaf-regions": "false"}):
+        k = compile_spn(native, spn, "float64", marginal=marginal, **dict(opts, **{"hip-kernel": "interpreter", "hip-compute-type": "float64"}))
+        src = k.source()
+        assert "compute f64" in src and ("features direct" in src) == (2 * leaves * regions > 48)
+        fused = (src.count("leafquad("), src.count("leafpair("), src.count("leafregion("))
+        assert fused == (want if "hip-interp-leaf-regions" not in opts else (0, 0, 0)), src[:2000]
+        got = run(k, X)
+        assert got.dtype == np.float64
+        assert np.abs(got - want64).max() <= F64_TOL, opts
+
+
 _LOAD_ORDER_SCRIPT = r"""
 import os, sys
 import numpy as np
