@@ -88,6 +88,7 @@ struct Emitter {
     uint32_t fa = 0, fb = UINT32_MAX;  // one feature, or a pair with a joint table
     uint32_t rowsA = 1, rowsB = 1;
     uint32_t base = 0, stride = 1;     // pool offset of the unit's table; entries per index (the siblings, padded to an even count)
+    uint32_t plane = 0;                // sibling planes: elements from one sibling's table to the next (then stride is 1); 0 = siblings side by side
   };
   struct FusedGroup {
     std::vector<uint32_t> products;                    // the siblings
@@ -257,6 +258,21 @@ struct Emitter {
     const size_t reads = (siblings + 1) / 2;
     return 2 * (reads | 1);
   }
+  // The other layout, sibling planes ("hip-table-planes"): every sibling's table on its own, entry j of sibling s at
+  // s * plane + j, read with one 4-byte (float) access per sibling, two siblings to an instruction. A wavefront's
+  // 4-byte accesses are served 32 lanes at a time from 32 banks, so lanes that read different entries of a table wait
+  // for each other only when the entries are a multiple of 32 apart; side by side, an 8-byte read covers 16 lanes at
+  // a time and entries 16 / reads apart collide. Simulated on the 100-feature discrete graph with uniform inputs:
+  // 41 % of the tables' LDS cycles are conflicts side by side (measured: 36 % of all LDS cycles), 24 % in planes.
+  // The distance between planes keeps every sibling's offset within what one read instruction with two offsets can
+  // name: 255 elements, or multiples of 64 elements.
+  static size_t fusedPlane(size_t siblings, size_t entries) {
+    if ((siblings - 1) * entries <= 255) return entries;
+    return (entries + 63) / 64 * 64;
+  }
+  size_t fusedElements(size_t siblings, size_t entries) const {
+    return o.tablePlanes && siblings > 1 ? siblings * fusedPlane(siblings, entries) : fusedStride(siblings) * entries;
+  }
 
   void planFusedGroups() {
     std::vector<uint32_t> parent(g.nodes.size(), UINT32_MAX);
@@ -317,7 +333,7 @@ struct Emitter {
     auto total = [&] {
       size_t t = other;
       for (const auto& G : fusedGroups)
-        for (const auto& u : G.units) t += fusedStride(G.products.size()) * size_t(u.rowsA) * u.rowsB;
+        for (const auto& u : G.units) t += fusedElements(G.products.size(), size_t(u.rowsA) * u.rowsB);
       return t;
     };
     const size_t budget = size_t(o.tableBudgetGiven ? o.tableBudgetKiB : 96) * 1024 / (f64 ? 8 : 4);
@@ -328,7 +344,9 @@ struct Emitter {
         for (size_t k = 0; k < G.units.size(); ++k) {
           const FusedUnit& u = G.units[k];
           if (u.fb == UINT32_MAX) continue;
-          const size_t gain = fusedStride(G.products.size()) * (size_t(u.rowsA) * u.rowsB - u.rowsA - u.rowsB);
+          const size_t siblings = G.products.size();
+          const size_t joint = fusedElements(siblings, size_t(u.rowsA) * u.rowsB), apart = fusedElements(siblings, u.rowsA) + fusedElements(siblings, u.rowsB);
+          const size_t gain = joint > apart ? joint - apart : 0;
           if (gain > bestGain) bestGain = gain, bestG = &G, bestU = k;
         }
       if (!bestG) break;
@@ -359,17 +377,22 @@ struct Emitter {
     for (auto& G : fusedGroups)
       for (auto& u : G.units) {
         const size_t k = G.products.size();
-        u.stride = uint32_t(fusedStride(k));
+        const size_t entries = size_t(u.rowsA) * u.rowsB;
+        const bool planes = o.tablePlanes && k > 1;
+        u.stride = planes ? 1u : uint32_t(fusedStride(k));
+        u.plane = planes ? uint32_t(fusedPlane(k, entries)) : 0u;
         if (tablePool.size() % 2) tablePool.push_back(0.0);
         u.base = uint32_t(tablePool.size());
-        const size_t entries = size_t(u.rowsA) * u.rowsB;
-        tablePool.resize(tablePool.size() + entries * u.stride, 0.0);
+        tablePool.resize(tablePool.size() + (planes ? k * u.plane : entries * u.stride), 0.0);
         for (size_t j = 0; j < k; ++j) {
           const std::vector<double> a = padded(G.leafOf[j].at(u.fa));
           const std::vector<double> b = u.fb == UINT32_MAX ? std::vector<double>{0.0} : padded(G.leafOf[j].at(u.fb));
           for (size_t x = 0; x < a.size(); ++x)
-            for (size_t y = 0; y < b.size(); ++y) tablePool[u.base + (x * b.size() + y) * u.stride + j] = a[x] + b[y];
+            for (size_t y = 0; y < b.size(); ++y)
+              tablePool[planes ? u.base + j * u.plane + (x * b.size() + y) : u.base + (x * b.size() + y) * u.stride + j] = a[x] + b[y];
         }
+        // how far past the pool's end an index made of unclamped (clamped) bytes can read, counted from the unit's last
+        // element: with planes, the last sibling's table is the one at the end
         largestRow = std::max(largestRow, size_t(u.rowsB + 1) * u.stride);
         reach = std::max(reach, size_t(packedSaturation()) * size_t(u.rowsB + 1) * u.stride);
       }
@@ -385,7 +408,6 @@ struct Emitter {
   }
 
   unsigned extractions2 = 0;
-  static std::string byteSel(uint32_t f) { return "BYTE_" + std::to_string(f % 4); }
   // The byte of feature f as a value of its own.
   // Written as a volatile statement: these stay in program order, so an index exists only from where the generator
   // put it. Left to the compiler, the extractions are merged or moved to the top of the kernel, and hundreds of
@@ -417,22 +439,30 @@ struct Emitter {
            << ";\n";
     }
     body << "  const bool outside = (outsideBits & 0x80808080u) != 0u;\n";
-    // Clamp: one byte-wise minimum per feature, in place (the other bytes of the register are preserved). Written as
-    // instructions: from the equivalent C expression the compiler makes about six instructions per feature. Left out
-    // when even an index made of arbitrary bytes stays inside the kernel's LDS: what such a read returns is dropped.
+    // Clamp: every byte to its feature's length, the register put together again. Written as instructions, and none
+    // of them one that selects bytes by itself (SDWA): a SIMD overlaps nothing with those. Left out when even an index
+    // made of arbitrary bytes stays inside the kernel's LDS: what such a read returns is dropped.
     for (uint32_t c = 0; c * 4 < g.numFeatures; ++c) {
-      std::string clamp, operands;
-      unsigned operand = 1;
-      for (uint32_t j = 0; j < 4 && c * 4 + j < g.numFeatures; ++j) {
-        const uint32_t f = c * 4 + j;
-        if (!featTableLen[f]) continue;
-        clamp += std::string(clamp.empty() ? "" : "\\n\\t") + "v_min_u32_sdwa %0, %0, %" + std::to_string(operand++) + " dst_sel:BYTE_" + std::to_string(j) +
-                 " dst_unused:UNUSED_PRESERVE src0_sel:BYTE_" + std::to_string(j) + " src1_sel:DWORD\\n\\ts_nop 0";  // a partial write, then a wait state
-        operands += std::string(operands.empty() ? "" : ", ") + "\"s\"(" + std::to_string(featTableLen[f]) + "u)";
-      }
-      if (clamp.empty()) continue;
+      bool any = false;
+      for (uint32_t j = 0; j < 4 && c * 4 + j < g.numFeatures; ++j) any = any || featTableLen[c * 4 + j];
+      if (!any) continue;
       body << "  unsigned PK" << c << " = R[" << c << "];\n";
-      if (clampPacked) body << "  asm(\"" << clamp << "\" : \"+v\"(PK" << c << ") : " << operands << ");\n";
+      if (!clampPacked) continue;
+      std::string text, operands;
+      unsigned operand = 3;
+      for (int j = 3; j >= 0; --j) {   // %0 the result, %1 a byte, %2 the packed register
+        const uint32_t f = c * 4 + uint32_t(j);
+        const uint32_t len = f < g.numFeatures && featTableLen[f] ? featTableLen[f] : 255u;
+        text += j == 3 ? "v_lshrrev_b32 %1, 24, %2\\n\\t" : j == 0 ? "v_and_b32 %1, 0xff, %2\\n\\t" : "v_bfe_u32 %1, %2, " + std::to_string(8 * j) + ", 8\\n\\t";
+        std::string limit = std::to_string(len);
+        if (len > 64) {
+          limit = "%" + std::to_string(operand++);
+          operands += ", \"s\"(" + std::to_string(len) + "u)";
+        }
+        text += std::string("v_min_u32 ") + (j == 3 ? "%0" : "%1") + ", " + limit + ", %1" + (j == 3 ? "" : "\\n\\tv_lshl_or_b32 %0, %0, 8, %1") + (j ? "\\n\\t" : "");
+      }
+      body << "  {\n    unsigned spn_q, spn_t;\n    asm(\"" << text << "\" : \"=&v\"(spn_q), \"=&v\"(spn_t) : \"v\"(PK" << c << ")" << operands << ");\n    PK" << c
+           << " = spn_q;\n  }\n";
     }
     for (uint32_t f = 0; f < g.numFeatures && o.hoistFeatureValues; ++f)
       if (featOneHot[f]) emitFeatureValues(f, "");
@@ -539,23 +569,53 @@ struct Emitter {
       std::vector<std::string> adds;
       for (size_t q = b0; q < std::min(G.units.size(), b0 + batch); ++q) {
         const FusedUnit& u = G.units[q];
-        // LDS address of the unit's entry: table + (a * rowsB + b) * stride * sizeof(real_t), as one statement of two
-        // or three instructions: a multiply per feature that takes its byte straight out of the packed register, and
-        // an add that brings in the table's address, so that every read of the unit is this register plus a
-        // constant offset. (Left to the compiler, the address of nearly every read got an add of its own.)
+        // LDS address of the unit's entry: table + (a * rowsB + b) * stride * sizeof(real_t), as one statement: the bytes
+        // of the two features are taken out of their packed registers, a 16-bit multiply-add makes the joint index and
+        // another one scales it and brings in the table's address, so that every read of the unit is this register plus
+        // a constant offset. (Left to the compiler, the address of nearly every read got an add of its own.)
+        // None of these is an SDWA, DPP or 24-bit-multiply instruction: on gfx950 a SIMD issues one of those in the
+        // time of about four plain instructions and overlaps nothing with it, while the ones used here issue every
+        // other cycle when they alternate with the additions of the wavefront beside them (measured with two
+        // wavefronts per SIMD: v_add_f32 alternating with v_mul_u32_u24_sdwa 2.2 ns per instruction, with v_bfe_u32
+        // or v_mad_u32_u16 1.05 ns).
         const std::string idx = "a" + std::to_string(extractions2++);
-        const std::string sel = " dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:";
         const size_t unitBytes = size_t(u.base) * realBytes;
+        std::string operands;   // scalar operands of the statement, numbered from `next`
+        unsigned nextOperand = u.fb != UINT32_MAX ? 4 : 2;
+        // A small integer is written into the instruction; anything else takes a register of the kind asked for.
+        auto constant = [&](size_t value, const char* kind) {
+          if (value <= 64) return std::to_string(value);
+          operands += std::string(", \"") + kind + "\"(" + std::to_string(value) + "u)";
+          return "%" + std::to_string(nextOperand++);
+        };
+        auto extract = [&](const char* dst, const char* src, uint32_t f) {
+          const unsigned byte = f % 4;
+          if (byte == 0) return std::string("v_and_b32 ") + dst + ", 0xff, " + src + "\\n\\t";
+          if (byte == 3) return std::string("v_lshrrev_b32 ") + dst + ", 24, " + src + "\\n\\t";
+          return std::string("v_bfe_u32 ") + dst + ", " + src + ", " + std::to_string(8 * byte) + ", 8\\n\\t";
+        };
+        const size_t strideBytes = size_t(u.stride) * realBytes;
         if (u.fb != UINT32_MAX) {
-          body << "  unsigned " << idx << ", " << idx << "b;\n  asm volatile(\"v_mul_u32_u24_sdwa %0, %2, %4" << sel << byteSel(u.fa) << " src1_sel:DWORD\\n\\t"
-               << "v_mul_u32_u24_sdwa %1, %3, %5" << sel << byteSel(u.fb) << " src1_sel:DWORD\\n\\tv_add3_u32 %0, %0, %1, %6\" : \"=&v\"(" << idx << "), \"=&v\"("
-               << idx << "b) : \"v\"(PK" << u.fa / 4 << "), \"v\"(PK" << u.fb / 4 << "), \"s\"(" << size_t(u.rowsB) * u.stride * realBytes << "u), \"s\"("
-               << u.stride * realBytes << "u), \"s\"(spn_tab_lds + " << unitBytes << "u));\n";
+          std::string text = extract("%0", "%2", u.fa) + extract("%1", "%3", u.fb);
+          text += "v_mad_u32_u16 %0, %0, " + constant(u.rowsB, "s") + ", %1\\n\\t";
+          const std::string scale = constant(strideBytes, "s");   // an instruction reads one scalar register at most
+          operands += std::string(", \"") + (strideBytes <= 64 ? "s" : "v") + "\"(spn_tab_lds + " + std::to_string(unitBytes) + "u)";
+          text += "v_mad_u32_u16 %0, %0, " + scale + ", %" + std::to_string(nextOperand++);
+          body << "  unsigned " << idx << ", " << idx << "b;\n  asm volatile(\"" << text << "\" : \"=&v\"(" << idx << "), \"=&v\"(" << idx << "b) : \"v\"(PK"
+               << u.fa / 4 << "), \"v\"(PK" << u.fb / 4 << ")" << operands << ");\n";
         } else {
-          body << "  unsigned " << idx << ";\n  asm volatile(\"v_mul_u32_u24_sdwa %0, %1, %2" << sel << byteSel(u.fa) << " src1_sel:DWORD\\n\\tv_add_u32 %0, %3, %0\" : \"=&v\"("
-               << idx << ") : \"v\"(PK" << u.fa / 4 << "), \"s\"(" << u.stride * realBytes << "u), \"s\"(spn_tab_lds + " << unitBytes << "u));\n";
+          std::string text = extract("%0", "%1", u.fa);
+          const std::string scale = constant(strideBytes, "s");
+          operands += std::string(", \"") + (strideBytes <= 64 ? "s" : "v") + "\"(spn_tab_lds + " + std::to_string(unitBytes) + "u)";
+          text += "v_mad_u32_u16 %0, %0, " + scale + ", %" + std::to_string(nextOperand++);
+          body << "  unsigned " << idx << ";\n  asm volatile(\"" << text << "\" : \"=&v\"(" << idx << ") : \"v\"(PK" << u.fa / 4 << ")" << operands << ");\n";
         }
-        for (size_t j = 0; j < k; j += 2) {
+        for (size_t j = 0; j < k && u.plane; ++j) {   // sibling planes: one value per read (the compiler pairs the reads into instructions with two offsets)
+          const std::string r = "r" + std::to_string(extractions2++);
+          body << "  const real_t " << r << " = *reinterpret_cast<const __attribute__((address_space(3))) real_t*>(" << idx << " + " << j * u.plane * realBytes << "u);\n";
+          adds.push_back("  " + next(j) + " += " + r + ";\n");
+        }
+        for (size_t j = 0; j < k && !u.plane; j += 2) {
           const std::string r = "r" + std::to_string(extractions2++);
           const std::string address = idx + " + " + std::to_string(j * realBytes) + "u";
           if (u.stride == 1) {
@@ -1438,23 +1498,26 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
 
   if (waveTile) {
     // Four values, each saturated (at 255, or with packed rows at the longest table's length: either is outside every
-    // table), into the four bytes of a register: one instruction per value (a minimum whose result goes into one byte
-    // of the destination and leaves the others alone). On this hardware a vector instruction must not read a register
-    // in the cycle after an instruction wrote part of it (the compiler's hazard pass, which does not look into assembler
-    // statements, keeps one wait state between the two): two registers are packed in turns, or idle cycles put between.
-    const std::string sat = std::to_string(e.packedRows ? e.packedSaturation() : 255u) + "u";
-    auto one = [](const char* dst, unsigned src, unsigned byte, unsigned satOperand) {
-      return std::string("v_min_u32_sdwa ") + dst + ", %" + std::to_string(src) + ", %" + std::to_string(satOperand) + " dst_sel:BYTE_" + std::to_string(byte) +
-             " dst_unused:" + (byte ? "UNUSED_PRESERVE" : "UNUSED_PAD") + " src0_sel:DWORD src1_sel:DWORD\\n\\t";
+    // table), into the four bytes of a register: a minimum per value and a shift-and-or per further byte, two registers
+    // in turns so that no instruction waits for the one before it. The one-instruction form, a minimum that writes one
+    // byte of its destination (SDWA), is the slower one on gfx950: a SIMD overlaps nothing with such an instruction.
+    const unsigned satValue = e.packedRows ? e.packedSaturation() : 255u;
+    const bool satInline = satValue <= 64;
+    auto sat = [&](unsigned operand) { return satInline ? std::to_string(satValue) : "%" + std::to_string(operand); };
+    const std::string satOperand = satInline ? std::string() : ", \"s\"(" + std::to_string(satValue) + "u)";
+    // dst = min(value 3) << 24 | min(value 2) << 16 | min(value 1) << 8 | min(value 0); values are operands first .. first + 3.
+    auto step = [&](const char* dst, const char* tmp, unsigned first, unsigned k, unsigned satOp) {
+      const std::string m = std::string("v_min_u32 ") + (k == 0 ? dst : tmp) + ", " + sat(satOp) + ", %" + std::to_string(first + 3 - k) + "\\n\\t";
+      return k == 0 ? m : m + "v_lshl_or_b32 " + dst + ", " + dst + ", 8, " + tmp + "\\n\\t";
     };
-    s << "static __device__ __forceinline__ unsigned spn_pack4(unsigned a, unsigned b, unsigned c, unsigned d) {\n  unsigned q;\n  asm(\"";
-    for (unsigned k = 0; k < 4; ++k) s << one("%0", 1 + k, k, 5) << "s_nop 0" << (k < 3 ? "\\n\\t" : "");
-    s << "\"\n      : \"=&v\"(q) : \"v\"(a), \"v\"(b), \"v\"(c), \"v\"(d), \"s\"(" << sat << "));\n  return q;\n}\n";
+    s << "static __device__ __forceinline__ unsigned spn_pack4(unsigned a, unsigned b, unsigned c, unsigned d) {\n  unsigned q, t;\n  asm(\"";
+    for (unsigned k = 0; k < 4; ++k) s << step("%0", "%1", 2, k, 6);
+    s << "\"\n      : \"=&v\"(q), \"=&v\"(t) : \"v\"(a), \"v\"(b), \"v\"(c), \"v\"(d)" << satOperand << ");\n  return q;\n}\n";
     s << "static __device__ __forceinline__ void spn_pack8(unsigned& p, unsigned& q, unsigned a0, unsigned a1, unsigned a2, unsigned a3, unsigned b0, unsigned b1, "
-         "unsigned b2, unsigned b3) {\n  asm(\"";
-    for (unsigned k = 0; k < 4; ++k) s << one("%0", 2 + k, k, 10) << one("%1", 6 + k, k, 10);
-    s << "s_nop 0\"\n      : \"=&v\"(p), \"=&v\"(q) : \"v\"(a0), \"v\"(a1), \"v\"(a2), \"v\"(a3), \"v\"(b0), \"v\"(b1), \"v\"(b2), \"v\"(b3), \"s\"(" << sat
-      << "));\n}\n";
+         "unsigned b2, unsigned b3) {\n  unsigned t, w;\n  asm(\"";
+    for (unsigned k = 0; k < 4; ++k) s << step("%0", "%2", 4, k, 12) << step("%1", "%3", 8, k, 12);
+    s << "\"\n      : \"=&v\"(p), \"=&v\"(q), \"=&v\"(t), \"=&v\"(w) : \"v\"(a0), \"v\"(a1), \"v\"(a2), \"v\"(a3), \"v\"(b0), \"v\"(b1), \"v\"(b2), \"v\"(b3)"
+      << satOperand << ");\n}\n";
   }
   if (e.vectorRows) {
     s << "static __device__ __forceinline__ void spn_load_row(const feat_t* __restrict__ in, unsigned long long i, feat_t (&x)[SPN_F]) {\n";
@@ -1569,8 +1632,10 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
   // Without an explicit option the tile is staged when the kernel is closer to the HBM bound
   // than to the VALU bound (about 6.4e12 B/s against 6e13 lane-operations/s on MI355X).
   const double tHbm = double(rowBytes + realBytes) / 6.4e12, tValu = double(g.stats.issueSlotsMin()) / 6.0e13;
+  // Static LDS besides the tables: float64 kernels keep their exp2/log2 tables and the leaves' pattern tables there.
+  const size_t ldsOther = (e.f64 ? (64 + 512 + 13) * sizeof(double) : 0) + e.cTables.size() * realBytes;
   const bool wantStaged = o.gpuSharedMem < 0 ? tHbm > 0.5 * tValu : o.gpuSharedMem == 1;
-  const bool staged = !waveTile && !g.isTask && wantStaged && e.vectorRows && tileBytes % 16 == 0 && tileBytes + ldsTables <= 64 * 1024;
+  const bool staged = !waveTile && !g.isTask && wantStaged && e.vectorRows && tileBytes % 16 == 0 && tileBytes + ldsTables + ldsOther <= 64 * 1024;
   js.stagedInput = staged;
   // Blocks with next to no set-up take one tile each; blocks that stage tables stay resident.
   js.oneTilePerBlock = js.tableEntries <= 256;

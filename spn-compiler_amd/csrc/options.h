@@ -53,6 +53,7 @@ struct CompileOptions {
   int interpStagedLong = -1;                   // "hip-interp-staged-features": lds|spill (-1 = automatic): tier of the staged input features
   long interpLongRange = -1;                   // "hip-interp-long-range": values living longer than this many instructions go to the long-lived pool (-1 = automatic)
   int packedRows = -1;                         // "hip-packed-rows": wide rows of small integer features stay packed four to a register and the table leaves of sibling products are evaluated together (1), not (0), decided per kernel (-1)
+  bool tablePlanes = true;                     // "hip-table-planes": with packed rows, the tables of sibling products lie one after the other (4-byte reads, fewer LDS bank conflicts) instead of side by side per entry
   int oneHotMaxDomain = 2;                     // "hip-one-hot-max-domain": with packed rows, table leaves over at most this many categories are evaluated as multiply-adds on the vector unit instead of LDS reads
   bool nanMasks = true;                        // "hip-nan-masks": with marginalisation in log space, a Gaussian leaf of a missing (NaN) feature is zeroed by a bitwise AND with a per-feature mask instead of a select per leaf
   int gaussExpanded = -1;                      // "hip-gauss-expanded": float64 log-space kernels evaluate a Gaussian leaf inside a product as A x^2 + B x + C on per-feature x^2, x and 1 (zeroed for a missing feature): three multiply-adds per leaf and no mask, two without marginalisation (-1 = where the expansion keeps 1e-11, see emit_hip.cpp)

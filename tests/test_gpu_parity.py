@@ -473,12 +473,12 @@ def test_packed_rows_on_the_discrete_configuration(native, variant, cfg):
     assert all(np.isneginf(got[r]) for r in (5, 6, 7, 8, 9)) and np.isfinite(got[10])
 
 
-@pytest.mark.parametrize("opts", [{}, {"hip-prefetch-rows": "false"}, {"hip-hoist-feature-values": "false"}, {"hip-fused-batch": 0}],
-                         ids=["default", "no-prefetch", "no-hoist", "unbatched"])
+@pytest.mark.parametrize("opts", [{}, {"hip-prefetch-rows": "false"}, {"hip-hoist-feature-values": "false"}, {"hip-fused-batch": 0}, {"hip-table-planes": "true"}],
+                         ids=["default", "no-prefetch", "no-hoist", "unbatched", "planes"])
 def test_packed_rows_with_long_tables(native, opts):
     """One sum over nine products of 32 categorical leaves, one feature with 120 categories: the padding that would make
-    unclamped packed bytes safe is too large here, so the kernel clamps every byte to its table's length (a minimum
-    written into one byte of the register, with the wait state that such a partial write needs). Inputs outside the
+    unclamped packed bytes safe is too large here, so the kernel clamps every byte to its table's length and puts the
+    register together again. Inputs outside the
     ranges, next to them and far away, give log 0."""
     from spnc.structure import Categorical, Product, Sum
     rng = np.random.default_rng(17)
@@ -496,9 +496,10 @@ def test_packed_rows_with_long_tables(native, opts):
     X[8, 5] = domains[5]
     X[9, 31] = 2 ** 31 - 1
     X[10, :] = [d - 1 for d in domains]
-    k = compile_spn(native, spn, "int32", marginal=False, **dict(opts, **{"hip-packed-rows": "true"}))
+    planes = opts.get("hip-table-planes") == "true"   # the siblings' tables one after the other: the padding stays small, nothing is clamped
+    k = compile_spn(native, spn, "int32", marginal=False, **dict({"hip-table-planes": "false"}, **dict(opts, **{"hip-packed-rows": "true"})))
     src = k.source()
-    assert "unsigned PK0 = R[0]" in src and "v_min_u32_sdwa %0, %0, %1 dst_sel:BYTE_0" in src   # packed rows, bytes clamped
+    assert "unsigned PK0 = R[0]" in src and ("PK0 = spn_q;" in src) == (not planes)   # packed rows, bytes clamped
     got = run(k, X)
     check_f32(got, oracle_model(spn, "int32"), X, False)
     assert all(np.isneginf(got[r]) for r in range(3, 10)) and np.isfinite(got[10]) and np.isfinite(got[:3]).all()

@@ -1,8 +1,8 @@
 """The kernel body that the generator emits for packed rows, run on the CPU: its text is cut out of a generated kernel,
-the assembler statements are rewritten as the C they stand for (byte selects, partial register writes, three-operand
-adds), the result is compiled for the host and compared with the oracle. This checks the generator's logic (tables,
-offsets, polynomials, range test) without a GPU; what only the hardware can show (wait states between partial register
-writes, LDS behaviour) is left to the GPU tests."""
+the assembler statements are rewritten as the C they stand for (bit fields, shift-and-or, 16-bit
+multiply-adds), the result is compiled for the host and compared with the oracle. This checks the generator's logic (tables,
+offsets, polynomials, range test) without a GPU; what only the hardware can show (LDS behaviour, the order of memory
+operations) is left to the GPU tests."""
 import ctypes
 import os
 import re
@@ -49,15 +49,16 @@ def _instruction(line, names):
         return f"{v[0]} = __builtin_fma({v[1]}, {v[2]}, {v[3]});"
     if op == "v_lshl_add_u32":
         return f"{v[0]} = (({v[1]}) << {v[2]}) + ({v[3]});"
-    if op in ("v_mul_u32_u24_sdwa", "v_min_u32_sdwa"):
-        a, b = _select(v[1], mods.get("src0_sel")), _select(v[2], mods.get("src1_sel"))
-        value = f"(({a} & 0xffffffu) * ({b} & 0xffffffu))" if op.startswith("v_mul") else f"(({a}) < ({b}) ? ({a}) : ({b}))"
-        sel = mods.get("dst_sel", "DWORD")
-        if sel == "DWORD":
-            return f"{v[0]} = {value};"
-        shift = 8 * int(sel[-1])
-        keep = f"({v[0]} & ~(255u << {shift}))" if mods.get("dst_unused") == "UNUSED_PRESERVE" else "0u"
-        return f"{v[0]} = {keep} | ((({value}) & 255u) << {shift});"
+    if op == "v_min_u32":
+        return f"{v[0]} = ({v[1]}) < ({v[2]}) ? ({v[1]}) : ({v[2]});"
+    if op == "v_lshl_or_b32":
+        return f"{v[0]} = (({v[1]}) << {v[2]}) | ({v[3]});"
+    if op == "v_and_b32":
+        return f"{v[0]} = ({v[1]}) & ({v[2]});"
+    if op == "v_lshrrev_b32":
+        return f"{v[0]} = ({v[2]}) >> {v[1]};"
+    if op == "v_mad_u32_u16":   # 16-bit factors, 32-bit sum
+        return f"{v[0]} = (({v[1]}) & 0xffffu) * (({v[2]}) & 0xffffu) + ({v[3]});"
     if op == "v_add3_u32":
         return f"{v[0]} = {v[1]} + {v[2]} + {v[3]};"
     if op == "v_add_u32":
@@ -118,7 +119,8 @@ extern "C" void eval_rows(const int* in, real_t* out, long n) {
   }
 }
 """ % (", [] {}" if templated else "")
-    assert ("s\"(%du)" % saturation) in source   # the value rows are saturated at when they are packed
+    # the value rows are saturated at when they are packed: written into the instruction when it is small enough for that
+    assert ("v_min_u32 %%0, %d, %%5" % saturation if saturation <= 64 else "\"s\"(%du)" % saturation) in source
     cpp, so = tmp_path / (tag + ".cpp"), tmp_path / (tag + ".so")
     cpp.write_text(text)
     subprocess.check_call([CLANG, "-O1", "-shared", "-fPIC", "-std=c++17", "-ffp-contract=fast", "-w", "-o", str(so), str(cpp)])
@@ -138,8 +140,9 @@ needs_clang = pytest.mark.skipif(not os.path.isfile(CLANG), reason="host build o
 @needs_clang
 @pytest.mark.parametrize("opts", [{}, {"hip-one-hot-max-domain": 3}, {"hip-one-hot-max-domain": 5, "hip-hoist-feature-values": "false"},
                                   {"hip-one-hot-max-domain": 0, "hip-fused-batch": 0}, {"hip-joint-tables": "false", "hip-prefetch-rows": "false"},
-                                  {"hip-table-budget-kib": 24}, {"hip-compute-type": "float64"}],
-                         ids=["default", "quadratic", "one-hot-5", "all-lds", "no-joint", "small-budget", "float64"])
+                                  {"hip-table-budget-kib": 24}, {"hip-compute-type": "float64"}, {"hip-table-planes": "false"},
+                                  {"hip-table-planes": "false", "hip-compute-type": "float64"}],
+                         ids=["default", "quadratic", "one-hot-5", "all-lds", "no-joint", "small-budget", "float64", "side-by-side", "side-by-side-float64"])
 @pytest.mark.parametrize("cfg", ["c3", "c3_deep"])
 def test_packed_rows_body_on_the_host(native, tmp_path, cfg, opts):
     from spnc import synthetic as syn
@@ -165,8 +168,11 @@ def test_packed_rows_body_on_the_host(native, tmp_path, cfg, opts):
 
 
 @needs_clang
-def test_packed_rows_body_with_clamped_bytes_on_the_host(native, tmp_path):
-    """A feature with 120 categories makes the padding for unclamped bytes too large: the bytes are clamped in place."""
+@pytest.mark.parametrize("planes", [False, True], ids=["side-by-side", "planes"])
+def test_packed_rows_body_with_clamped_bytes_on_the_host(native, tmp_path, planes):
+    """A feature with 120 categories makes the padding for unclamped bytes too large when the siblings' values lie side
+    by side: the bytes are clamped in place. With the siblings' tables in planes the padding stays small and no byte is
+    clamped."""
     from spnc.structure import Categorical, Product, Sum
     rng = np.random.default_rng(17)
     domains = [120] + [int(d) for d in rng.integers(2, 7, 31)]
@@ -175,10 +181,11 @@ def test_packed_rows_body_with_clamped_bytes_on_the_host(native, tmp_path):
     spn = Sum([float(v) for v in rng.dirichlet(np.ones(9))], products)
     X = np.column_stack([rng.integers(0, d, 2000) for d in domains]).astype(np.int32)
     X[3, 0], X[4, 0], X[5, 0], X[6, 0], X[7, 0], X[8, 5], X[9, 31] = 120, 127, 128, 255, 256, domains[5], 2 ** 31 - 1
-    k = compile_spn(native, spn, "int32", marginal=False, **{"hip-packed-rows": "true"})
+    k = compile_spn(native, spn, "int32", marginal=False, **{"hip-packed-rows": "true", "hip-table-planes": "true" if planes else "false"})
     src = k.source()
     os.remove(k.fileName())
-    assert "v_min_u32_sdwa %0, %0, %1 dst_sel:BYTE_0" in src
+    # the clamp of the long feature's byte, its limit in a register
+    assert ("PK0 = spn_q;" not in src) if planes else ("v_min_u32 %1, %3, %1" in src and "PK0 = spn_q;" in src)
     got = run_host(host_library(src, 120, tmp_path, "long"), X, np.float32)
     ref = ev.ll_closed_f64(oracle_model(spn, "int32"), X, marginal=False)
     assert np.array_equal(np.isneginf(got), np.isneginf(ref)) and all(np.isneginf(got[r]) for r in range(3, 10))
