@@ -295,8 +295,11 @@ def cpu_baseline(name, cfg, spn, x_host):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # Defaults: the chip takes 25-40 ms of load to settle (power management: launch 2 of the 100-feature discrete
+    # configuration runs 0.60 ms, launches 5-8 0.75 ms, from about launch 40 on 0.58 ms; the 16-feature Gaussian one
+    # falls from 1.9 to 1.57 ms over its first 12 launches). A job of many batches runs in the settled state.
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", default="c1", choices=["c1", "c2", "c3", "c3_deep", "c4", "c5", "c5_f64", "c4_f64"])
     ap.add_argument("--n", type=int, default=0, help="override the number of samples")
     ap.add_argument("--no-others", action="store_true", help="measure only the selected configuration")

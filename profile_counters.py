@@ -22,6 +22,7 @@ import tempfile
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 BENCH = os.path.join(ROOT, "bench.py")
+STEPS, WARMUP = 50, 50   # bench.py's own defaults: the timed launches start once the chip has settled under the load
 KERNELS = {"c1": "spn_kernel", "c2": "spn_kernel", "c3": "spn_kernel", "c4": "spn_interp_kernel", "c5": "spn_kernel", "c5_f64": "spn_kernel", "c4_f64": "spn_interp_kernel"}
 SQ_SETS = [
     "SQ_INSTS_VALU SQ_INSTS_SALU SQ_INSTS_SMEM SQ_INSTS_LDS SQ_WAVE_CYCLES SQ_BUSY_CYCLES SQ_ACTIVE_INST_VALU SQ_WAIT_INST_ANY",
@@ -52,6 +53,12 @@ def kernel_stats(con):
     for r in rows[:4]:
         lines.append("%-46s %6d %12.0f %12d %12d %6.1f%%" % (r[0][:46], r[1], r[2], r[3], r[4], 100.0 * r[5] / total))
     return lines, rows
+
+
+def timed_launches(con, like, steps):
+    """Average duration (ns) of the kernel's last `steps` dispatches: the ones bench.py times, after its warm-up launches."""
+    rows = con.execute("select end-start from kernels where name like ? order by start desc limit ?", (like, steps)).fetchall()
+    return sum(r[0] for r in rows) / len(rows), len(rows)
 
 
 def counters(con, like):
@@ -88,7 +95,7 @@ def main():
         name = KERNELS[cfg]
         like = "%" + name + "%"
         common = ["--config", cfg, "--no-others", "--fast-inputs"]
-        con, stdout, shown = rocprof(work, "stats_" + cfg, ["--kernel-trace", "--stats"], common + ["--steps", "20"])
+        con, stdout, shown = rocprof(work, "stats_" + cfg, ["--kernel-trace", "--stats"], common + ["--steps", str(STEPS), "--warmup", str(WARMUP)])
         line = json.loads(stdout.strip().splitlines()[-1])
         roof, n = line["roofline"], line["config"]["samples"]
         stats, rows = kernel_stats(con)
@@ -97,7 +104,8 @@ def main():
                 "Every pass is one rocprofv3 run of bench.py (inputs drawn on the device: --fast-inputs); figures are read from the sqlite",
                 "database rocprofv3 writes (kernels: name, count, avg/min/max of end-start; pmc_events: counter sums per dispatch).", "",
                 "$ " + shown] + stats
-        avg_ns = next(r[2] for r in rows if name in r[0])
+        avg_ns, timed = timed_launches(con, like, STEPS)
+        stats.append("%-46s %6d %12.0f   (the last %d calls: the launches bench.py times, after %d warm-up launches)" % (name[:46], timed, avg_ns, timed, WARMUP))
         per_launch = {}
         for counter in ("FETCH_SIZE", "WRITE_SIZE"):
             con, _, shown = rocprof(work, counter + "_" + cfg, ["--pmc", counter], common + ["--steps", "5"])
@@ -106,7 +114,7 @@ def main():
             text += ["$ " + shown, "%-46s %-12s per-dispatch=%.1f units" % (name, counter, value)]
         hbm_bytes = (per_launch["FETCH_SIZE"] * units["FETCH_SIZE"] + per_launch["WRITE_SIZE"] * units["WRITE_SIZE"]) * 1024
         algorithmic = roof["bytes_per_sample"] * n
-        text += ["", "bench.py, same run as the kernel trace: %.4g samples/s, launch %.4f ms (HIP events); rocprofv3 average %.4f ms."
+        text += ["", "bench.py, same run as the kernel trace: %.4g samples/s, launch %.4f ms (HIP events); rocprofv3 average of the same launches %.4f ms."
                  % (line["value"], roof["launch_ms"], avg_ns / 1e6),
                  "roofline bound %s, achieved %s of %s %s = %s." % (roof["bound"], roof["achieved"], roof["peak"], roof["unit"], roof["frac"]),
                  "Counter calibration (profiles/copy_kernel_counters.txt): FETCH_SIZE x %.3f, WRITE_SIZE x %.3f give KiB of HBM traffic."
