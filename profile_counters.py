@@ -99,13 +99,13 @@ def main():
         line = json.loads(stdout.strip().splitlines()[-1])
         roof, n = line["roofline"], line["config"]["samples"]
         stats, rows = kernel_stats(con)
+        avg_ns, timed = timed_launches(con, like, STEPS)
+        stats.append("%-46s %6d %12.0f   (the last %d calls: the launches bench.py times, after %d warm-up launches)" % (name[:46], timed, avg_ns, timed, WARMUP))
         text = ["Kernel %s, workload %s" % (name, line["config"]["workload"]),
                 "MI355X (gfx950), %d samples per launch. Made by: python3 profile_counters.py %s" % (n, cfg),
                 "Every pass is one rocprofv3 run of bench.py (inputs drawn on the device: --fast-inputs); figures are read from the sqlite",
                 "database rocprofv3 writes (kernels: name, count, avg/min/max of end-start; pmc_events: counter sums per dispatch).", "",
                 "$ " + shown] + stats
-        avg_ns, timed = timed_launches(con, like, STEPS)
-        stats.append("%-46s %6d %12.0f   (the last %d calls: the launches bench.py times, after %d warm-up launches)" % (name[:46], timed, avg_ns, timed, WARMUP))
         per_launch = {}
         for counter in ("FETCH_SIZE", "WRITE_SIZE"):
             con, _, shown = rocprof(work, counter + "_" + cfg, ["--pmc", counter], common + ["--steps", "5"])
