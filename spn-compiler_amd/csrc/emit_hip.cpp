@@ -70,6 +70,8 @@ struct Emitter {
   // product) is read from a table of 2^k entries in LDS, indexed by the pattern of present features, and is the
   // value the multiply-adds accumulate onto: one LDS read per product instead of one multiply-add per leaf.
   std::vector<double> cTables;
+  std::vector<double> standIn;   // per feature: the value a missing input is replaced by when products take the leaves' offsets from a table
+  bool marginalOffsets = false;
   std::map<std::vector<uint32_t>, std::string> patternNames;  // features of a product (in leaf order) -> variable with the pattern
   std::vector<bool> featUsed;
   std::vector<bool> featPrepared;
@@ -163,9 +165,36 @@ struct Emitter {
     return sum <= 1e-11;
   }
 
+  // Missing features of float kernels, in products that evaluate their Gaussian leaves themselves ("hip-marginal-offsets"):
+  // a missing value is replaced once per feature by a stand-in (the middle of the means of the feature's leaves), every
+  // leaf is then evaluated without a select, and what the leaves over missing features added to the product, which
+  // depends only on which of its features are missing, is taken off again with one value from a table in LDS (one
+  // entry per pattern of missing features, four leaves to a table). A select per leaf is a quarter of such a
+  // product's instructions. What is added and taken off again costs half an ulp of the running sum per leaf, so only
+  // leaves whose value at the stand-in is small take part (at most 8 in magnitude, at most 32 per product together:
+  // 1e-5 of error at worst); the others, narrow leaves far from the stand-in, keep their select.
+  bool decideMarginalOffsets() {
+    standIn.assign(g.numFeatures, 0.0);
+    if (!(g.supportMarginal && logSpace && !f64 && o.marginalOffsets && o.marginalTablesKiB > 0)) return false;
+    std::vector<double> lo(g.numFeatures, HUGE_VAL), hi(g.numFeatures, -HUGE_VAL);
+    for (const auto& n : g.nodes)
+      if (n.kind == NodeKind::Gaussian) lo[n.feature] = std::min(lo[n.feature], n.mean), hi[n.feature] = std::max(hi[n.feature], n.mean);
+    for (uint32_t f = 0; f < g.numFeatures; ++f)
+      if (lo[f] <= hi[f]) standIn[f] = double(float(0.5 * (lo[f] + hi[f])));
+    return true;
+  }
+  // What a Gaussian leaf over a missing feature adds to its product when it is evaluated at the feature's stand-in.
+  double offsetOf(const GraphNode& leaf) const {
+    const double den = -(1.0 / (2.0 * leaf.stddev * leaf.stddev)) * scale;
+    const double coef = (-std::log(leaf.stddev) + -0.5 * std::log(2 * M_PI)) * scale;
+    const double d = standIn[leaf.feature] - leaf.mean;
+    return den * d * d + coef;
+  }
+
   void prepare() {
     expandedGauss = decideExpandedGauss();
     laneConstants = expandedGauss && o.laneConstants;
+    marginalOffsets = decideMarginalOffsets();
     featTableLen.assign(g.numFeatures, 0);
     featGauss.assign(g.numFeatures, false);
     featUsed.assign(g.numFeatures, false);
@@ -870,6 +899,8 @@ struct Emitter {
           body << "  const real_t gx" << f << " = g" << f << ";\n";
         body << "  const real_t gq" << f << " = gx" << f << " * gx" << f << ";\n";
       }
+      if (featGauss[f] && marginalOffsets)
+        body << "  const bool gn" << f << " = g" << f << " != g" << f << ";\n  const real_t gz" << f << " = gn" << f << " ? " << lit(standIn[f]) << " : g" << f << ";\n";
       if (featGauss[f] && nanMasks()) {
         // All ones, or zero when the feature is missing. The empty assembler statement hides where the value came from:
         // otherwise the compiler turns every AND with it back into a select.
@@ -1088,10 +1119,56 @@ struct Emitter {
       emitExpandedLeaves(i, leaves, acc, fold);
       return;
     }
+    // Offsets of the leaves over missing features, four leaves to a table, while the tables fit; smallest offsets first.
+    std::vector<std::string> corrections;
+    std::vector<bool> viaTable(leaves.size(), false);
+    if (marginalOffsets && !leaves.empty()) {
+      std::vector<size_t> order(leaves.size());
+      for (size_t k = 0; k < order.size(); ++k) order[k] = k;
+      std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) { return std::fabs(offsetOf(g.nodes[leaves[a]])) < std::fabs(offsetOf(g.nodes[leaves[b]])); });
+      double together = 0.0;
+      std::vector<size_t> chosen;
+      for (size_t k : order) {
+        const double offset = std::fabs(offsetOf(g.nodes[leaves[k]]));
+        if (offset > 8.0 || together + offset > 32.0) break;
+        together += offset;
+        chosen.push_back(k);
+      }
+      std::sort(chosen.begin(), chosen.end());
+      if ((cTables.size() + 16 * ((chosen.size() + 3) / 4)) * sizeof(float) > size_t(o.marginalTablesKiB) * 1024) chosen.clear();
+      for (size_t lo = 0; lo < chosen.size(); lo += 4) {
+        std::vector<uint32_t> feats;
+        std::vector<double> ks;
+        for (size_t j = lo; j < std::min(chosen.size(), lo + 4); ++j) {
+          const auto& leaf = g.nodes[leaves[chosen[j]]];
+          viaTable[chosen[j]] = true;
+          emitFeaturePrep(leaf.feature);
+          feats.push_back(leaf.feature);
+          ks.push_back(offsetOf(leaf));
+        }
+        auto pattern = patternNames.find(feats);
+        if (pattern == patternNames.end()) {
+          const std::string name = "pm" + std::to_string(patternNames.size());
+          body << "  const unsigned " << name << " = ";
+          for (size_t q = 0; q < feats.size(); ++q) body << (q ? " | " : "") << "(gn" << feats[q] << " ? 0u : " << (1u << q) << "u)";
+          body << ";\n";
+          pattern = patternNames.emplace(feats, name).first;
+        }
+        const size_t base = cTables.size();
+        for (unsigned mask = 0; mask < (1u << feats.size()); ++mask) {   // bit q set: feature q is there
+          double sum = 0.0;
+          for (size_t q = 0; q < feats.size(); ++q)
+            if (!(mask >> q & 1u)) sum -= ks[q];
+          cTables.push_back(sum);
+        }
+        corrections.push_back("SPN_CTAB[" + std::to_string(base) + "u + " + pattern->second + "]");
+      }
+    }
     for (size_t k = 0; k < leaves.size(); ++k) {
       const auto& leaf = g.nodes[leaves[k]];
       emitFeaturePrep(leaf.feature);
-      const std::string x = "g" + std::to_string(leaf.feature);
+      const bool offsets = viaTable[k];
+      const std::string x = (offsets ? "gz" : "g") + std::to_string(leaf.feature);
       const double den = -(1.0 / (2.0 * leaf.stddev * leaf.stddev)) * scale;
       const double coef = (-std::log(leaf.stddev) + -0.5 * std::log(2 * M_PI)) * scale;
       // The weight a parent sum folded into this product rides on the first leaf's constant; with masks it would be
@@ -1101,7 +1178,7 @@ struct Emitter {
       body << "  const real_t " << d << " = " << x << " - " << lit(leaf.mean) << ";\n";
       if (nanMasks())
         body << "  const real_t " << t << " = " << masked(std::string(fma) + d + ", " + d + ", " + lit(coef / den) + ")", leaf.feature) << ";\n";
-      else if (g.supportMarginal)
+      else if (g.supportMarginal && !offsets)
         body << "  const real_t " << t << " = (" << x << " != " << x << ") ? " << lit(extra) << " : " << fma << d << ", " << d << ", "
              << lit(coef / den + extra) << ");\n";
       else
@@ -1110,6 +1187,7 @@ struct Emitter {
       else body << "  const real_t " << a << " = " << fma << t << ", " << lit(den) << ", " << acc << ");\n";
       acc = a;
     }
+    for (const std::string& c : corrections) acc = "(" + acc + " + " + c + ")";
     if (nanMasks() && fold != 0.0 && !leaves.empty()) body << "  const real_t " << v(i) << " = " << acc << " + " << lit(fold) << ";\n";
     else body << "  const real_t " << v(i) << " = " << acc << ";\n";
   }
@@ -1341,6 +1419,12 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
     const size_t bigTile = size_t(512) * U * rowBytes;
     if (tHbmAuto > tValuAuto && bigTile % 16 == 0 && bigTile + size_t(js.tableEntries) * realBytes <= 64 * 1024) js.blockSize = 512;
   }
+  // Float kernels without tables: blocks of 512 threads, so that a SIMD always holds an even number of wavefronts. Full
+  // rate instructions issue from two wavefronts in turns, and an odd number of wavefronts loses part of that (v_add_f32
+  // alone: 1.09 ns per instruction at two wavefronts per SIMD, 1.39 at three, 1.08 at four). Measured: 16 Gaussian
+  // features 1.63 -> 1.60 ms, the same with 20 % missing values (95 registers, five wavefronts of 256-thread blocks or
+  // four of 512-thread ones) 1.62 -> 1.56 ms. Double kernels are slower that way (4.34 -> 4.89 ms) and stay at 256.
+  if (o.blockSize == 0 && !e.f64 && e.logSpace && !g.isTask && js.tableEntries == 0 && e.vectorRows) js.blockSize = 512;
   js.libraryMath = !e.log2Dom;
   js.doubleConstants = e.f64;
   // Wide rows of 32-bit integer features read only by table leaves: a lane that fetches its own row touches 64 cache
@@ -1456,8 +1540,10 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
          "  unsigned hi;\n"
          "  asm(\"v_lshl_add_u32 %0, %1, 14, %2\" : \"=v\"(hi) : \"v\"(ni), \"v\"(t.w[1]));\n"
          "  t.w[1] = hi;\n"
-         "  real_t p = SPN_POLY[0];\n"
-         "  p = __builtin_fma(p, r, SPN_POLY[1]);\n  p = __builtin_fma(p, r, SPN_POLY[2]);\n"
+         // 2^r - 1 = r (c1 + c2 r + c3 r^2 + c4 r^3) for |r| <= 1/128: the next term, c5 r^5, is below 4e-14 of the
+         // result, a thousand times below what the results are held to (1e-10), and one multiply-add per call less.
+         "  real_t p = SPN_POLY[1];\n"
+         "  p = __builtin_fma(p, r, SPN_POLY[2]);\n"
          "  p = __builtin_fma(p, r, SPN_POLY[3]);\n  p = __builtin_fma(p, r, SPN_POLY[4]);\n"
          "  return __builtin_fma(t.d, p * r, t.d);\n}\n";
     s << "static __device__ " << mathAttr << " real_t spn_log2(real_t x) {\n"
@@ -1467,8 +1553,8 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
          "  const unsigned j = (hi >> 12) & 255u;\n"
          "  c.u = (c.u & 0x000fffffffffffffull) | 0x3ff0000000000000ull;\n"
          "  const real_t u = __builtin_fma(c.d, SPN_LOG2_TABLE[2 * j], -1.0);\n"
-         "  real_t p = SPN_POLY[5];\n"
-         "  p = __builtin_fma(p, u, SPN_POLY[6]);\n  p = __builtin_fma(p, u, SPN_POLY[7]);\n"
+         // log2(1 + u) = u (l1 + l2 u + ... + l5 u^4) for 0 <= u < 1/256: the next term, l6 u^6, is below 1e-15.
+         "  real_t p = SPN_POLY[7];\n"
          "  p = __builtin_fma(p, u, SPN_POLY[8]);\n  p = __builtin_fma(p, u, SPN_POLY[9]);\n"
          "  p = __builtin_fma(p, u, SPN_POLY[10]);\n  p = __builtin_fma(p, u, SPN_POLY[11]);\n"
          "  const real_t r = __builtin_fma(u, p, SPN_LOG2_TABLE[2 * j + 1] + (real_t)e);\n"
@@ -1610,9 +1696,9 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
   if (e.log2Dom && e.f64)
     s << "  for (unsigned t = threadIdx.x; t < 64; t += SPN_BLOCK) spn_exp2_lds[t] = spn_exp2_table[t];\n"
          "  for (unsigned t = threadIdx.x; t < 512; t += SPN_BLOCK) spn_log2_lds[t] = spn_log2_table[t];\n"
-         "  if (threadIdx.x < 13) spn_poly_lds[threadIdx.x] = spn_poly[threadIdx.x];\n"
-      << (e.cTables.empty() ? "" : "  for (unsigned t = threadIdx.x; t < SPN_NCTAB; t += SPN_BLOCK) spn_ctab_lds[t] = spn_ctab[t];\n")
-      << "  __syncthreads();\n";
+         "  if (threadIdx.x < 13) spn_poly_lds[threadIdx.x] = spn_poly[threadIdx.x];\n";
+  if (!e.cTables.empty()) s << "  for (unsigned t = threadIdx.x; t < SPN_NCTAB; t += SPN_BLOCK) spn_ctab_lds[t] = spn_ctab[t];\n";
+  if ((e.log2Dom && e.f64) || !e.cTables.empty()) s << "  __syncthreads();\n";
   if (js.tableEntries && js.tablesInLds) {
     s << "  __shared__ __attribute__((aligned(32))) real_t tab[SPN_NTAB];\n"
          "  for (unsigned t = threadIdx.x; t < SPN_NTAB; t += SPN_BLOCK) tab[t] = spn_tables[t];\n"

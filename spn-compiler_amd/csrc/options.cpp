@@ -112,6 +112,8 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
       o.hoistFeatureValues = parseBool(val);
     } else if (key == "hip-packed-rows") {
       o.packedRows = parseBool(val) ? 1 : 0;
+    } else if (key == "hip-marginal-offsets") {
+      o.marginalOffsets = parseBool(val);
     } else if (key == "hip-table-planes") {
       o.tablePlanes = parseBool(val);
     } else if (key == "hip-one-hot-max-domain") {

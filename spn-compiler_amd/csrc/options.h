@@ -53,6 +53,7 @@ struct CompileOptions {
   int interpStagedLong = -1;                   // "hip-interp-staged-features": lds|spill (-1 = automatic): tier of the staged input features
   long interpLongRange = -1;                   // "hip-interp-long-range": values living longer than this many instructions go to the long-lived pool (-1 = automatic)
   int packedRows = -1;                         // "hip-packed-rows": wide rows of small integer features stay packed four to a register and the table leaves of sibling products are evaluated together (1), not (0), decided per kernel (-1)
+  bool marginalOffsets = true;                 // "hip-marginal-offsets": float kernels replace a missing feature by a stand-in value, evaluate the Gaussian leaves of a product without selects and take what the leaves over missing features added off again with one table value per product
   bool tablePlanes = true;                     // "hip-table-planes": with packed rows, the tables of sibling products lie one after the other (4-byte reads, fewer LDS bank conflicts) instead of side by side per entry
   int oneHotMaxDomain = 2;                     // "hip-one-hot-max-domain": with packed rows, table leaves over at most this many categories are evaluated as multiply-adds on the vector unit instead of LDS reads
   bool nanMasks = true;                        // "hip-nan-masks": with marginalisation in log space, a Gaussian leaf of a missing (NaN) feature is zeroed by a bitwise AND with a per-feature mask instead of a select per leaf

@@ -332,6 +332,7 @@ Graph buildGraph(const RawQuery& q) {
   g.nodes.back().uses++;
   GraphStats& st = g.stats;
   uint64_t leafSelect = q.supportMarginal ? 1 : 0;
+  uint64_t ownSelects = 0, ownCorrections = 0;
   for (const auto& n : g.nodes) {
     uint64_t k = n.children.size();
     st.maxFanIn = std::max<uint32_t>(st.maxFanIn, uint32_t(k));
@@ -362,6 +363,10 @@ Graph buildGraph(const RawQuery& q) {
           uint64_t own = 0;  // Gaussian children read by this product only
           for (uint32_t c : n.children) own += g.nodes[c].kind == NodeKind::Gaussian && g.nodes[c].uses == 1 ? 1 : 0;
           st.fusedMin += std::min<uint64_t>(own, k ? k - 1 : 0);
+          // Marginal queries: such leaves need no select of their own. A missing feature is replaced once by a stand-in
+          // value, and what the leaves over missing features add to the product is taken off with one table value per
+          // four leaves (one add each).
+          if (leafSelect && own) ownSelects += own, ownCorrections += (own + 3) / 4;
         }
         break;
       case NodeKind::Sum: {
@@ -383,6 +388,14 @@ Graph buildGraph(const RawQuery& q) {
         break;
       }
     }
+  }
+  if (ownSelects) {   // instead of a select per leaf: an add per correction, and per Gaussian feature the stand-in and its bit of the pattern
+    std::vector<bool> gaussianFeature(g.numFeatures, false);
+    for (const auto& n : g.nodes)
+      if (n.kind == NodeKind::Gaussian) gaussianFeature[n.feature] = true;
+    uint64_t perFeature = 0;
+    for (bool b : gaussianFeature) perFeature += b ? 2 : 0;
+    if (ownCorrections + perFeature < ownSelects) st.flopsMin = st.flopsMin - ownSelects + ownCorrections + perFeature;
   }
   // Sums over a complete outer product of two operand vectors: M sums share the ordered child list
   // [prod(a_0,b_0), ..., prod(a_NA-1,b_NB-1)] and nothing else reads those products. Since

@@ -81,7 +81,8 @@ struct GraphStats {
   uint32_t maxFanIn = 0;
   uint32_t serializedNodes = 0;  // before dropping unreachable nodes and merging duplicates
   // Algorithmic work per sample: cheaper of pairwise tree (k==2) and n-ary LSE (k>=3) per sum,
-  // 4 flops per Gaussian, 0 per table leaf, +1 select per leaf when marginal.
+  // 4 flops per Gaussian, 0 per table leaf, +1 select per leaf when marginal (Gaussian leaves that one product alone
+  // reads: one add per four leaves and two selects per feature instead, which is what the float kernels do).
   uint64_t flopsMin = 0, transMin = 0, flopsPairwise = 0, transPairwise = 0;
   // Multiply-add pairs among flopsMin that one fused instruction computes in log space: a Gaussian leaf's
   // (d*d)*den + coef, and the add of a product for every Gaussian child that only this product reads

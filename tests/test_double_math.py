@@ -49,14 +49,15 @@ def test_double_exp2_log2_against_libm(native, tmp_path, marginal):
     got = np.array([lib.spn_exp2(float(x)) for x in xs])
     want = np.exp2(xs)
     normal = want > 1e-300
-    assert np.max(np.abs(got[normal] - want[normal]) / want[normal]) < 1e-15
+    # the polynomial stops at the fourth power of the remainder (at most 1/128): 4e-14 of the result, against 1e-10 that results are held to
+    assert np.max(np.abs(got[normal] - want[normal]) / want[normal]) < 5e-14
     assert np.all(got[~normal] <= 1e-299)
     assert lib.spn_exp2(float("-inf")) == 0.0 and lib.spn_exp2(-5000.0) == 0.0
     assert marginal or np.isnan(lib.spn_exp2(float("nan")))
     ss = np.concatenate([rng.uniform(1, 700, 20000), np.exp2(rng.uniform(-1000, 1000, 4000)), [1.0, 2.0, 0.5, 1.4142135623730951, 0.7071067811865476]])
     got = np.array([lib.spn_log2(float(s)) for s in ss])
     want = np.log2(ss)
-    assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-3)) < 1e-15
+    assert np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-3)) < 3e-15   # the polynomial stops at the fifth power of u < 1/256: 1e-15
     near = rng.uniform(1.0, 1.001, 5000)            # sums dominated by one term: absolute accuracy matters
     assert max(abs(lib.spn_log2(float(s)) - np.log2(s)) for s in near) < 1e-17 * 50
     assert lib.spn_log2(1.0) == 0.0 and lib.spn_log2(0.0) == float("-inf")

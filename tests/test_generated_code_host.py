@@ -137,9 +137,11 @@ def test_golden_models_on_the_host(native, tmp_path, name, opts):
                                        ("c5", {"hip-compute-type": "float64", "hip-lane-constants": "false"}),
                                        ("c5", {"hip-compute-type": "float64", "hip-marginal-tables-kib": 0}),
                                        ("c5", {"hip-compute-type": "float64", "hip-marginal-tables-kib": 3}),
-                                       ("c2", {"hip-compute-type": "float64"}), ("c2", {"hip-compute-type": "float64", "hip-lane-constants": "false"})],
+                                       ("c2", {"hip-compute-type": "float64"}), ("c2", {"hip-compute-type": "float64", "hip-lane-constants": "false"}),
+                                       ("c5", {"hip-marginal-offsets": "false"}), ("c5", {"maxTaskSize": 150}), ("c5", {"hip-marginal-tables-kib": 1})],
                          ids=["c1", "c1-cut", "c2", "c2-cut", "c5", "c5-f64", "c5-f64-cut", "c5-f64-selects", "c3-cut", "c5-f64-factored",
-                              "c5-f64-scalar-constants", "c5-f64-no-pattern-tables", "c5-f64-few-pattern-tables", "c2-f64", "c2-f64-scalar-constants"])
+                              "c5-f64-scalar-constants", "c5-f64-no-pattern-tables", "c5-f64-few-pattern-tables", "c2-f64", "c2-f64-scalar-constants",
+                              "c5-selects", "c5-cut", "c5-few-offset-tables"])
 def test_benchmark_graphs_on_the_host(native, tmp_path, cfg, opts):
     from spnc import synthetic as syn
     c = syn.CONFIGS[cfg]
