@@ -1727,6 +1727,9 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
   js.oneTilePerBlock = js.tableEntries <= 256;
   if (staged || waveTile) js.inputAlign = 16;
   if (waveTile) js.oneTilePerBlock = false;
+  if (o.ldsBallastKiB > 0 && !g.isTask)   // claimed, touched once so that it stays, never read for a result
+    s << "  __shared__ unsigned spn_ballast[" << o.ldsBallastKiB * 256 << "];\n  if (n == ~0ull) spn_ballast[threadIdx.x] = 1u;\n"
+         "  if (n == ~0ull - 1ull) out[0] = (real_t)spn_ballast[threadIdx.x ^ 1u];\n";
   s << "  const unsigned long long tile = (unsigned long long)SPN_BLOCK * SPN_U;\n";
   if (waveTile)
     s << "  typedef unsigned int spn_v4 __attribute__((ext_vector_type(4)));\n"

@@ -138,6 +138,9 @@ CompileOptions parseOptions(const std::map<std::string, std::string>& kv) {
     } else if (key == "hip-table-group-window") {
       o.tableGroupWindow = parseInt(key, val);
       if (o.tableGroupWindow < 0) throw std::runtime_error("hip-table-group-window must not be negative");
+    } else if (key == "hip-lds-ballast-kib") {
+      o.ldsBallastKiB = parseInt(key, val);
+      if (o.ldsBallastKiB < 0 || o.ldsBallastKiB > 150) throw std::runtime_error("hip-lds-ballast-kib must be in [0,150]");
     } else if (key == "hip-table-pad-kib") {
       o.tablePadKiB = parseInt(key, val);
       if (o.tablePadKiB < 0 || o.tablePadKiB > 64) throw std::runtime_error("hip-table-pad-kib must be in [0,64]");

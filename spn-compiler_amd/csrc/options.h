@@ -39,6 +39,7 @@ struct CompileOptions {
   bool groupedTables = true;                   // "hip-grouped-tables": tables read with the same index are interleaved in blocks of four columns and fetched up to four per read
   int tableGroupMinReads = 200;                // "hip-table-group-min-reads": graphs with fewer table reads per sample keep plain tables
   int tableGroupWindow = 96;                   // "hip-table-group-window": tables of a group are used within this many table uses of each other
+  int ldsBallastKiB = 0;                       // "hip-lds-ballast-kib": LDS a block claims without using it, which caps the blocks (and wavefronts) a CU holds; for measurement
   int tablePadKiB = 18;                        // "hip-table-pad-kib": LDS beyond the table budget that blocks of four columns may take (unused columns)
   int tableBudgetKiB = 62;                     // "hip-table-budget-kib": LDS the table pool may grow to when leaves are paired into joint tables
   bool tableBudgetGiven = false;               // without the option, kernels on packed rows pair up to 96 KiB (measured on the 100-feature discrete graph: 0.78 ms at 62 KiB, 0.75 ms at 80, 0.74 ms at 96 with leaves over three categories in tables too)
