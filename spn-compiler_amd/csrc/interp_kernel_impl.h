@@ -445,17 +445,18 @@ struct MatrixSteps {
   // e: product of this step, e1: product of the next step (made one step ago, used one step from now).
   static __device__ __forceinline__ void run(const float* ea, const float* eb, const float (*A)[2], float4v& d0, float4v& d1, float e,
                                              float e1) {
+    static_assert(K != 0 || KEND > 2, "the first step of a chain is the one that writes the accumulators whole");
     if constexpr (K + 2 < KEND) {
       float e2;
       if constexpr (K == 0) {
         // The two wait states in front separate the first matrix instruction from the vector instructions
-        // that made its operands.
+        // that made its operands. The first step adds onto the constant 0, so the accumulators need no clearing.
         asm volatile(
             "s_nop 1\n\t"
-            "v_mfma_f32_4x4x1_16b_f32 %0, %3, %5, %0 cbsz:4 abid:%8\n\t"
+            "v_mfma_f32_4x4x1_16b_f32 %0, %3, %5, 0 cbsz:4 abid:%8\n\t"
             "v_mul_f32 %2, %6, %7\n\t"
-            "v_mfma_f32_4x4x1_16b_f32 %1, %4, %5, %1 cbsz:4 abid:%8"
-            : "+v"(d0), "+v"(d1), "=&v"(e2)
+            "v_mfma_f32_4x4x1_16b_f32 %1, %4, %5, 0 cbsz:4 abid:%8"
+            : "=&v"(d0), "=&v"(d1), "=&v"(e2)
             : "v"(A[K / 16][0]), "v"(A[K / 16][1]), "v"(e), "v"(ea[(K + 2) / NB]), "v"(eb[(K + 2) % NB]), "n"(K % 16), "v"(e1));
       } else {
         // No operand of this statement was written by the statement before it (the product comes from two
@@ -542,7 +543,7 @@ __device__ __forceinline__ void matrixChainAndStore(const float* ea, const float
                                                     const Slots<float, SPILL>& S) {
   typedef Math<float, LOG2> Mt;
   constexpr int M = 8, K = NA * NB;
-  float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+  float4v d0, d1;   // written whole by the chain's first step
   SPN_PRIO_CHAIN();
   MatrixSteps<0, K, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
   SPN_PRIO_LATENCY();
@@ -662,13 +663,12 @@ __device__ __forceinline__ R leafOperands(code_ptr ip, long rec, const R* x, R* 
     }
     e[i] = acc;
   }
-  R ma = R(-__builtin_huge_val()), mb = R(-__builtin_huge_val());
+  // The maxima start from the lowest finite value, which keeps them finite when every product is impossible.
+  R ma = Mt::lowest(), mb = Mt::lowest();
 #pragma unroll
   for (int r = 0; r < NA; ++r) ma = rmax(ma, e[r]);
 #pragma unroll
   for (int c = 0; c < NB; ++c) mb = rmax(mb, e[NA + c]);
-  ma = rmax(ma, Mt::lowest());
-  mb = rmax(mb, Mt::lowest());
 #pragma unroll
   for (int r = 0; r < NA; ++r) ea[r] = Mt::exp(e[r] - ma);
 #pragma unroll
@@ -745,7 +745,7 @@ __device__ __forceinline__ code_ptr leafRegionMatrixG(code_ptr ip, const Head& h
 // instruction; the program builder fuses sums only where the weights keep the largest entry of such a vector above 2^-90.
 template <int NA, int NB>
 __device__ __forceinline__ void rawChain(const float* ea, const float* eb, const float (*A)[2], float* v) {
-  float4v d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+  float4v d0, d1;   // written whole by the chain's first step
   SPN_PRIO_CHAIN();
   MatrixSteps<0, NA * NB, NB>::run(ea, eb, A, d0, d1, ea[0] * eb[0], ea[1 / NB] * eb[1 % NB]);
   SPN_PRIO_LATENCY();
@@ -790,7 +790,8 @@ __device__ __forceinline__ code_ptr leafPairMatrix(code_ptr ip, const Head& h, c
 #pragma unroll
   for (int side = 0; side < 2; ++side) {
     float ea[N], eb[N];
-    base += leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + side * RECS, x + side * 2 * G, ea, eb);
+    const float maxima = leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + side * RECS, x + side * 2 * G, ea, eb);
+    base = side == 0 ? maxima : base + maxima;   // not 0 + maxima: that is an instruction (it turns -0 into +0)
     rawChain<N, N>(ea, eb, side == 0 ? A1 : A2, side == 0 ? va : vb);
   }
   matrixChainAndStore<LOG2, SPILL, 8, 8>(va, vb, AT, base, (w1 >> 8) & 1u, h, DST, SCALE, tierD, (w1 >> 11) & 1u, S);
@@ -848,7 +849,8 @@ __device__ __forceinline__ code_ptr leafQuadMatrix(code_ptr ip, const Head& h, c
     for (int side = 0; side < 2; ++side) {
       const int region = 2 * pair + side;
       float ea[N], eb[N];
-      base += leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + region * RECS, x + region * 2 * G, ea, eb);
+      const float maxima = leafOperands<LOG2, N, N, G, MARGINAL>(ip, REC + region * RECS, x + region * 2 * G, ea, eb);
+      base = region == 0 ? maxima : base + maxima;   // not 0 + maxima: that is an instruction (it turns -0 into +0)
       rawChain<N, N>(ea, eb, AL[region], v[side]);
     }
     if (pair == 0) {
