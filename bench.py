@@ -138,6 +138,7 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None, fast_inpu
     wall = time.perf_counter() - t0
     launch_ms = sum(s.elapsed_time(e) for s, e in zip(starts, ends)) / steps
     finite = bool(torch.isfinite(out[: min(n, 1 << 20)]).all().item())
+    head = out[: min(n, 1 << 12)].cpu().numpy()   # what the CPU baseline leg compares its own results with
 
     bytes_per_sample = cfg["features"] * info["bytes_per_feature"] + info["bytes_per_result"]
     flops, trans = info["flops_min"], info["trans_min"]
@@ -192,11 +193,11 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None, fast_inpu
             roof["sustained_over_published"] = round(sustained / valu_peak, 4)
             roof["frac_of_sustained"] = round(slots * n / sustained / t_launch, 4)
     if f64:
-        # A float64 exp or log is not one quarter-rate instruction as in float32 but a routine of its own: about 11
-        # double-rate instructions and one LDS read here. Priced at that cost the same launch reads:
-        slots_real = flops - info["fused_min"] + 10 * trans
-        roof["issue_slots_per_sample_exp_log_at_11"] = slots_real
-        roof["frac_exp_log_at_11"] = round(slots_real * n / valu_peak / t_launch, 4)
+        # A float64 exp or log is not one quarter-rate instruction as in float32 but a routine of its own: nine
+        # double-rate instructions, three to six integer ones and one LDS read here. Priced at the nine the same launch reads:
+        slots_real = flops - info["fused_min"] + 8 * trans
+        roof["issue_slots_per_sample_exp_log_at_9"] = slots_real
+        roof["frac_exp_log_at_9"] = round(slots_real * n / valu_peak / t_launch, 4)
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by what a plain copy of known
     # size reads on the same counters): written to profiles/traffic.json by profile_counters.py together with a hash of
     # the kernel's code and launch size, so that an entry measured on another kernel is not passed on.
@@ -215,7 +216,7 @@ def measure(name, n, steps, warmup, torch, device, extra_options=None, fast_inpu
         "roofline": roof, "compile_s": round(compile_s, 2), "nodes": info["num_nodes"], "finite": finite,
         "kernel_key": kernel_key(kernel, n),
     }
-    return res, kernel, x_host, cfg, spn
+    return res, kernel, x_host, cfg, spn, head
 
 
 def host_path(kernel, x_host, torch):
@@ -246,9 +247,10 @@ def host_path(kernel, x_host, torch):
     return res
 
 
-def cpu_baseline(name, cfg, spn, x_host):
+def cpu_baseline(name, cfg, spn, x_host, gpu_head=None):
     """The restated CPUCompiler-equivalent kernel, timed on this host on a bounded sample of the same inputs, on all
-    OpenMP threads and on one."""
+    OpenMP threads and on one. Its results for the first rows are also held against what the GPU kernel wrote for them
+    (`max_abs_diff_vs_gpu`; rows where both are minus infinity agree)."""
     sys.path.insert(0, ROOT)
     from oracle import c_oracle, cgen, spn_model as sm
     from xspn.serialization.binary.BinarySerialization import BinarySerializer
@@ -288,7 +290,16 @@ def cpu_baseline(name, cfg, spn, x_host):
         set_threads(1)
         one_rate, one_n = rate(1.5)
         set_threads(threads)
+        diff = None
+        if gpu_head is not None and len(gpu_head):
+            import numpy as np
+            ref = np.asarray(run(x_host[:len(gpu_head)]), dtype=np.float64)
+            got = np.asarray(gpu_head, dtype=np.float64)
+            both = np.isfinite(ref) & np.isfinite(got)
+            same_inf = (np.isneginf(ref) == np.isneginf(got)).all() and not np.isnan(got).any()
+            diff = float(np.abs(ref[both] - got[both]).max(initial=0.0)) if same_inf else float("inf")
     return {"value": all_rate, "unit": "samples/s", "cores": threads, "kind": "port", "one_thread_value": one_rate,
+            "max_abs_diff_vs_gpu": diff,
             "sample": f"first {all_n} rows of the same batch ({one_n} for the one-thread figure), one pass each; {how}"}
 
 
@@ -345,14 +356,14 @@ def main():
 
     def one(name):
         with contextlib.redirect_stdout(log):
-            res, kernel, x_host, cfg, spn = measure(name, args.n if name == args.config else 0, args.steps, args.warmup, torch, device, extra,
-                                                    args.fast_inputs)
+            res, kernel, x_host, cfg, spn, head = measure(name, args.n if name == args.config else 0, args.steps, args.warmup, torch, device, extra,
+                                                          args.fast_inputs)
         torch.cuda.empty_cache()
         if not args.no_host and name in ("c1", "c2"):
             with contextlib.redirect_stdout(log):
                 res["host_path"] = host_path(kernel, x_host, torch)
         if not args.no_cpu:
-            res["cpu_baseline"] = cpu_baseline(res["workload"], cfg, spn, x_host)
+            res["cpu_baseline"] = cpu_baseline(res["workload"], cfg, spn, x_host, head)
             if res.get("host_path") and res["cpu_baseline"]["value"] > 0:
                 # below 1: for data that starts in host memory, the host's own cores finish sooner than the trip over PCIe
                 res["host_path_vs_cpu_baseline"] = round(res["host_path"]["pageable_samples_per_s"] / res["cpu_baseline"]["value"], 3)
