@@ -154,3 +154,44 @@ def test_benchmark_graphs_on_the_host(native, tmp_path, cfg, opts):
     fin = np.isfinite(ref)
     assert np.array_equal(np.isneginf(got), np.isneginf(ref))
     assert np.abs(got[fin] - ref[fin]).max() <= (1e-4 if got.dtype == np.float32 else 1e-10)
+
+
+def _wide_marginal_products(seed=3):
+    """A sum over five products of eleven Gaussian leaves each, some of them narrow and far from the others (their value
+    at the stand-in for a missing feature is large, so they keep their select), with rows that miss none, some and all
+    of their features."""
+    from spnc.structure import Gaussian, Product, Sum
+    rng = np.random.default_rng(seed)
+    products = []
+    for _ in range(5):
+        leaves = []
+        for f in range(11):
+            narrow = rng.random() < 0.25
+            leaves.append(Gaussian(mean=float(rng.normal(0, 3 if narrow else 1)), stdev=float(rng.uniform(0.05, 0.2) if narrow else rng.uniform(0.5, 2.0)), scope=f))
+        products.append(Product(children=leaves))
+    spn = Sum([float(v) for v in rng.dirichlet(np.ones(5))], products)
+    X = rng.normal(0, 1.5, (600, 11)).astype(np.float32)
+    X[rng.random(X.shape) < 0.3] = np.nan
+    X[0, :] = np.nan
+    X[1, :10] = np.nan
+    X[2, 1:] = np.nan
+    X[3, :] = 0.25
+    return spn, X
+
+
+@pytest.mark.parametrize("opts", [{}, {"hip-marginal-offsets": "false"}, {"hip-marginal-tables-kib": 1}, {"maxTaskSize": 20}],
+                         ids=["offsets", "selects", "few-tables", "cut"])
+def test_missing_features_in_wide_products_on_the_host(native, tmp_path, opts):
+    spn, X = _wide_marginal_products()
+    k = compile_spn(native, spn, "float32", marginal=True, **dict(opts, **{"hip-kernel": "jit"}))
+    info, src = k.info(), k.source()
+    os.remove(k.fileName())
+    if not opts:
+        assert "SPN_CTAB[" in src and " != g" in src   # both forms in one kernel: table offsets, and selects for the narrow leaves
+    got = host_kernel(src, info, tmp_path)(X)
+    ref = ev.ll_closed_f64(oracle_model(spn, "float32"), X, marginal=True)
+    assert np.isfinite(ref).all() and abs(ref[0]) < 1e-12   # every feature missing: log 1
+    # the narrow leaves put results at -100 to -3000, where a float's own spacing is up to 2.4e-4: 1e-4 plus three such steps
+    assert (np.abs(got - ref) <= 1e-4 + 4e-7 * np.abs(ref)).all()
+    near = np.abs(ref) < 60
+    assert near.sum() > 50 and np.abs(got[near] - ref[near]).max() <= 1e-4

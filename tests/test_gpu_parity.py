@@ -505,6 +505,29 @@ def test_packed_rows_with_long_tables(native, opts):
     assert all(np.isneginf(got[r]) for r in range(3, 10)) and np.isfinite(got[10]) and np.isfinite(got[:3]).all()
 
 
+@pytest.mark.parametrize("opts", [{}, {"hip-marginal-offsets": "false"}, {"hip-marginal-tables-kib": 1}, {"maxTaskSize": 20, "hip-kernel": "jit"},
+                                  {"hip-kernel": "interpreter"}],
+                         ids=["offsets", "selects", "few-tables", "cut", "interpreter"])
+def test_missing_features_in_wide_products(native, opts):
+    """Products of eleven Gaussian leaves under one sum, a quarter of the leaves narrow and far from the others, rows that
+    miss none, some and all of their features: float kernels take what leaves over missing features add off again with a
+    table value per four leaves, and keep a select for the leaves whose value at the stand-in is large."""
+    from test_generated_code_host import _wide_marginal_products
+    spn, X = _wide_marginal_products()
+    X = np.tile(X, (9, 1))[:5000]
+    k = compile_spn(native, spn, "float32", marginal=True, **opts)
+    if not opts:
+        src = k.source()
+        assert "SPN_CTAB[" in src and " != g" in src
+    got = run(k, X)
+    ref = ev.ll_closed_f64(oracle_model(spn, "float32"), X, marginal=True)
+    assert got.dtype == np.float32 and np.isfinite(ref).all() and abs(got[0]) < 1e-6   # every feature missing: log 1
+    # the narrow leaves put results at -100 to -3000, where a float's own spacing is up to 2.4e-4: 1e-4 plus three such steps
+    assert (np.abs(got - ref) <= F32_TOL + 4e-7 * np.abs(ref)).all()
+    near = np.abs(ref) < 60
+    assert near.sum() > 400 and np.abs(got[near] - ref[near]).max() <= F32_TOL
+
+
 @pytest.mark.parametrize("dtype,marginal", [("uint8", False), ("int32", False), ("float32", True), ("float64", True)])
 def test_grouped_tables_feature_types_and_marginals(native, dtype, marginal):
     """Small graph, grouping forced: every feature has five or six table leaves (one index each), joint tables for the
