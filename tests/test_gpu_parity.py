@@ -506,8 +506,8 @@ def test_packed_rows_with_long_tables(native, opts):
 
 
 @pytest.mark.parametrize("opts", [{}, {"hip-marginal-offsets": "false"}, {"hip-marginal-tables-kib": 1}, {"maxTaskSize": 20, "hip-kernel": "jit"},
-                                  {"hip-kernel": "interpreter"}],
-                         ids=["offsets", "selects", "few-tables", "cut", "interpreter"])
+                                  {"hip-kernel": "interpreter"}, {"hip-samples-per-lane": 2}, {"hip-block-size": 256, "gpu-shared-mem": "true"}],
+                         ids=["offsets", "selects", "few-tables", "cut", "interpreter", "two-samples-per-lane", "staged-rows"])
 def test_missing_features_in_wide_products(native, opts):
     """Products of eleven Gaussian leaves under one sum, a quarter of the leaves narrow and far from the others, rows that
     miss none, some and all of their features: float kernels take what leaves over missing features add off again with a
