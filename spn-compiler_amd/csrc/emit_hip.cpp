@@ -1445,7 +1445,10 @@ JitSource emitHipSource(const Graph& g, const CompileOptions& o, const std::stri
       const size_t tables = js.tablesInLds ? size_t(js.tableEntries) * realBytes : 0;
       unsigned block = o.blockSize ? unsigned(o.blockSize) : 512u;
       while (!o.blockSize && block > 64 && tables + size_t(block / 64) * 64 * waveStride * 4 > 150 * 1024) block /= 2;
-      if (tables + size_t(block / 64) * 64 * waveStride * 4 <= 150 * 1024) {
+      // Packed rows address their tables inside LDS: a pool that is too large for LDS leaves the graph to the kernel with
+      // one index per feature (built below).
+      const bool tablesReachable = !e.packedRows || js.tableEntries == 0 || js.tablesInLds;
+      if (tablesReachable && tables + size_t(block / 64) * 64 * waveStride * 4 <= 150 * 1024) {
         waveTile = true;
         js.blockSize = block;
       }

@@ -505,6 +505,22 @@ def test_packed_rows_with_long_tables(native, opts):
     assert all(np.isneginf(got[r]) for r in range(3, 10)) and np.isfinite(got[10]) and np.isfinite(got[:3]).all()
 
 
+def test_discrete_graph_whose_tables_do_not_fit_lds(native):
+    """10 k nodes over 64 integer features: the table pool is too large for LDS, so the kernel reads its tables from
+    global memory with one index per feature (packed rows address their tables inside LDS and are not used)."""
+    from spnc import synthetic as syn
+    spn = syn.c3_spn(64, 33, sum_levels=3, inner_fan_in=(2, 9))
+    X = syn.c3_inputs(3000, 64, 33, data_seed=933)
+    X[5, :] = 77
+    X[6, 3] = 9
+    X[2999, 0] = -1
+    k = compile_spn(native, spn, "int32", marginal=False)
+    assert "unsigned PK0 = R[0]" not in k.source()
+    got = run(k, X)
+    check_f32(got, oracle_model(spn, "int32"), X, False)
+    assert np.isneginf(got[5]) and np.isneginf(got[6]) and np.isneginf(got[2999])
+
+
 @pytest.mark.parametrize("opts", [{}, {"hip-marginal-offsets": "false"}, {"hip-marginal-tables-kib": 1}, {"maxTaskSize": 20, "hip-kernel": "jit"},
                                   {"hip-kernel": "interpreter"}, {"hip-samples-per-lane": 2}, {"hip-block-size": 256, "gpu-shared-mem": "true"}],
                          ids=["offsets", "selects", "few-tables", "cut", "interpreter", "two-samples-per-lane", "staged-rows"])

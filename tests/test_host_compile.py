@@ -442,3 +442,14 @@ def test_max_task_size_cuts_the_graph_into_bounded_tasks(native, tmp_path, name,
                        k.bytesPerResult(), k.dataType())
     assert k2.info()["num_tasks"] == info["num_tasks"] and k2.info()["task_rows"] == info["task_rows"]
     os.remove(k.fileName())
+
+
+def test_discrete_graph_whose_tables_do_not_fit_lds(native):
+    """Packed rows address their tables inside LDS. A graph whose table pool is too large for LDS (10 k nodes over 64
+    features here) is built with one index per feature instead, and still compiles."""
+    from spnc import synthetic as syn
+    spn = syn.c3_spn(64, 33, sum_levels=3, inner_fan_in=(2, 9))
+    k = compile_spn(native, spn, "int32", marginal=False)
+    src = k.source()
+    os.remove(k.fileName())
+    assert "unsigned PK0 = R[0]" not in src and "spn_tab_lds" not in src and "const real_t* tab = spn_tables;" in src
