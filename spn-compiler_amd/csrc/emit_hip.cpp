@@ -183,12 +183,15 @@ struct Emitter {
       if (lo[f] <= hi[f]) standIn[f] = double(float(0.5 * (lo[f] + hi[f])));
     return true;
   }
-  // What a Gaussian leaf over a missing feature adds to its product when it is evaluated at the feature's stand-in.
-  double offsetOf(const GraphNode& leaf) const {
+  // What a Gaussian leaf over a missing feature adds to its product when it is evaluated at the feature's stand-in,
+  // from the constants as the kernel holds them (rounded to float: with a very narrow leaf next to the stand-in the
+  // rounding of its mean alone moves the value by more than the results may differ). `folded`: the log-weight that rides
+  // on this leaf's constant (the first leaf of a product); it stays in the product when the feature is missing.
+  double offsetOf(const GraphNode& leaf, double folded = 0.0) const {
     const double den = -(1.0 / (2.0 * leaf.stddev * leaf.stddev)) * scale;
     const double coef = (-std::log(leaf.stddev) + -0.5 * std::log(2 * M_PI)) * scale;
-    const double d = standIn[leaf.feature] - leaf.mean;
-    return den * d * d + coef;
+    const double d = double(float(standIn[leaf.feature])) - double(float(leaf.mean));
+    return double(float(den)) * (d * d + double(float(coef / den + folded / den))) - folded;
   }
 
   void prepare() {
@@ -1144,7 +1147,7 @@ struct Emitter {
           viaTable[chosen[j]] = true;
           emitFeaturePrep(leaf.feature);
           feats.push_back(leaf.feature);
-          ks.push_back(offsetOf(leaf));
+          ks.push_back(offsetOf(leaf, chosen[j] == 0 ? fold : 0.0));
         }
         auto pattern = patternNames.find(feats);
         if (pattern == patternNames.end()) {

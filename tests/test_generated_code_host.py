@@ -195,3 +195,31 @@ def test_missing_features_in_wide_products_on_the_host(native, tmp_path, opts):
     assert (np.abs(got - ref) <= 1e-4 + 4e-7 * np.abs(ref)).all()
     near = np.abs(ref) < 60
     assert near.sum() > 50 and np.abs(got[near] - ref[near]).max() <= 1e-4
+
+
+def _narrow_leaf_next_to_the_stand_in():
+    """Two products over two features; on feature 0 one leaf is very narrow (stddev 0.003) and sits 0.01 from the value
+    that stands in for a missing input (the middle of the two means). Its value there is small, so it goes through the
+    table, but it moves by 1e-4 when the mean moves by one float rounding: the table entry has to come from the rounded
+    constants the kernel computes with."""
+    from spnc.structure import Gaussian, Product, Sum
+    spn = Sum([0.3, 0.7], [Product(children=[Gaussian(mean=1.0, stdev=0.5, scope=0), Gaussian(mean=0.2, stdev=1.0, scope=1)]),
+                           Product(children=[Gaussian(mean=1.02, stdev=0.003, scope=0), Gaussian(mean=-0.4, stdev=0.8, scope=1)])])
+    rng = np.random.default_rng(8)
+    X = np.column_stack((rng.normal(1.01, 0.01, 400), rng.normal(0, 1, 400))).astype(np.float32)
+    X[::2, 0] = np.nan
+    X[::5, 1] = np.nan
+    return spn, X
+
+
+def test_narrow_leaf_next_to_the_stand_in_on_the_host(native, tmp_path):
+    spn, X = _narrow_leaf_next_to_the_stand_in()
+    k = compile_spn(native, spn, "float32", marginal=True, **{"hip-kernel": "jit"})
+    info, src = k.info(), k.source()
+    os.remove(k.fileName())
+    assert "SPN_CTAB[" in src and ") ? 0x" not in src   # both leaves of both products through tables, no select of a constant
+    got = host_kernel(src, info, tmp_path)(X)
+    ref = ev.ll_closed_f64(oracle_model(spn, "float32"), X, marginal=True)
+    missing = np.isnan(X[:, 0])
+    assert np.abs(got[missing] - ref[missing]).max() <= 2e-6   # nothing of the narrow leaf is left when its feature is missing
+    assert (np.abs(got - ref) <= 1e-4 + 4e-7 * np.abs(ref)).all()

@@ -505,6 +505,21 @@ def test_packed_rows_with_long_tables(native, opts):
     assert all(np.isneginf(got[r]) for r in range(3, 10)) and np.isfinite(got[10]) and np.isfinite(got[:3]).all()
 
 
+def test_narrow_leaf_next_to_the_stand_in(native):
+    """A very narrow Gaussian leaf 0.01 from the value that stands in for its feature when it is missing: the table entry
+    that takes the leaf's value off again comes from the rounded constants the kernel computes with (from the unrounded
+    ones it would be 3e-5 off)."""
+    from test_generated_code_host import _narrow_leaf_next_to_the_stand_in
+    spn, X = _narrow_leaf_next_to_the_stand_in()
+    k = compile_spn(native, spn, "float32", marginal=True, **{"hip-kernel": "jit"})
+    assert "SPN_CTAB[" in k.source()
+    got = run(k, X)
+    ref = ev.ll_closed_f64(oracle_model(spn, "float32"), X, marginal=True)
+    missing = np.isnan(X[:, 0])
+    assert np.abs(got[missing] - ref[missing]).max() <= 2e-6
+    assert (np.abs(got - ref) <= F32_TOL + 4e-7 * np.abs(ref)).all()
+
+
 def test_discrete_graph_whose_tables_do_not_fit_lds(native):
     """10 k nodes over 64 integer features: the table pool is too large for LDS, so the kernel reads its tables from
     global memory with one index per feature (packed rows address their tables inside LDS and are not used)."""
